@@ -53,8 +53,9 @@ typedef int kiln_marlin_status_t;
  * with the same name and argument order.  Differences, all documented:
  *   - A and C are bf16 (the reference wrapper's two casts, lib.rs:169,269, go away);
  *   - B and s are in the tile layout;
- *   - `workspace` must hold kiln_w4a16_workspace_bytes(m, n, k) bytes, zero on
- *     first use; every call leaves its counter region zero again (the
+ *   - `workspace` must hold kiln_w4a16_workspace_bytes(m, n, k) bytes (with overrides:
+ *     kiln_w4a16_workspace_bytes_tuned), its first kiln_w4a16_workspace_zeroed_bytes()
+ *     bytes zero on first use; every call leaves that counter region zero again (the
  *     reference's lock array has the same in/out contract, marlin_kernel.cu:177-180);
  *   - `stream` is a hipStream_t; thread_k (rows of K per block or K slice) and
  *     thread_n (columns per block) keep the reference's meaning as overrides of
@@ -69,11 +70,26 @@ kiln_marlin_status_t kiln_marlin_w4a16_gemm(
     int thread_k, int thread_n, int sms, int max_par);
 
 /*
- * Bytes of device workspace the GEMM entry points need for this shape.
- * Replaces the reference wrapper's fixed `(n / 128) * max_par` int32 sizing
- * (lib.rs:176-178).  Monotone in m, so sizing for the largest m is enough.
+ * Bytes of device workspace the GEMM entry points need for up to prob_m rows of this
+ * projection shape with the automatic plan (thread_k = thread_n = sms = -1).  Replaces the
+ * reference wrapper's fixed `(n / 128) * max_par` int32 sizing (lib.rs:176-178).
+ * The value is the largest need of any row count from 1 to prob_m, so it never decreases
+ * with prob_m: one workspace sized for the largest m a caller will issue serves every
+ * smaller call.  Only the first kiln_w4a16_workspace_zeroed_bytes() bytes (arrival
+ * counters) must be zero before the first call; every call leaves them zero again, and
+ * nothing else in the workspace carries state from one call to the next.
  */
 size_t kiln_w4a16_workspace_bytes(int prob_m, int prob_n, int prob_k);
+
+/* The same for a caller that passes plan overrides to kiln_marlin_w4a16_gemm (<= 0: automatic). */
+size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k,
+                                        int thread_k, int thread_n, int sms);
+
+/*
+ * Length of the workspace prefix that must be zero on first use (64 KiB of counters; the
+ * reference's whole lock array has that contract, marlin_kernel.cu:177-180, lib.rs:176-178).
+ */
+size_t kiln_w4a16_workspace_zeroed_bytes(void);
 
 /*
  * C = A * dequant(B, s) + sum_i scale_i * (A * lora_a_i^T) * lora_b_i^T.  Fuses what

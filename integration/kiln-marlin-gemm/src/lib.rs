@@ -6,7 +6,9 @@
 //!   * activations and output are bf16 end to end (no fp16 round trip);
 //!   * `b_packed` / `scales` carry the tile layout of the HIP kernels (same shapes,
 //!     `[k/16, 2n]` i32 and `[k/g, n]` f16; contents are opaque to callers);
-//!   * the workspace is sized by `kiln_w4a16_workspace_bytes`.
+//!   * the workspace is sized by `kiln_w4a16_workspace_bytes`, kept per (device, stream) and
+//!     grown on demand; only its counter prefix (`kiln_w4a16_workspace_zeroed_bytes`) is ever
+//!     cleared, once, when the buffer is allocated -- no memset rides in front of a GEMM.
 //! All arithmetic lives behind the C ABI declared in `include/kiln_w4a16.h`.
 //!
 //! Written without a Rust toolchain at hand: the storage accessors follow candle 0.10's
@@ -16,6 +18,8 @@
 use candle_core::{backend::BackendStorage, cuda_backend::cudarc::driver::DevicePtr, DType, Result, Tensor};
 use core::ffi::c_void;
 use half::{bf16, f16};
+use std::collections::HashMap;
+use std::sync::{Mutex, OnceLock};
 
 unsafe extern "C" {
     fn kiln_marlin_w4a16_gemm(
@@ -24,6 +28,7 @@ unsafe extern "C" {
         dev: i32, stream: *mut c_void, thread_k: i32, thread_n: i32, sms: i32, max_par: i32,
     ) -> i32;
     fn kiln_w4a16_workspace_bytes(prob_m: i32, prob_n: i32, prob_k: i32) -> usize;
+    fn kiln_w4a16_workspace_zeroed_bytes() -> usize;
     fn kiln_w4a16_quantize_and_pack(
         weight: *const f32, k: i32, n: i32, groupsize: i32,
         b_packed: *mut i32, scales_f16: *mut u16, dequant: *mut f32,
@@ -58,10 +63,9 @@ pub fn marlin_w4a16_gemm(a: &Tensor, b_packed: &Tensor, scales: &Tensor, groupsi
     if scales.dtype() != DType::F16 { candle_core::bail!("kiln-marlin-gemm: scales must be f16 (got {:?})", scales.dtype()); }
 
     let (a, b_packed, scales) = (a.contiguous()?, b_packed.contiguous()?, scales.contiguous()?);
-    let out = Tensor::zeros((m, n), DType::BF16, a.device())?;
-    // zero on first use; every call leaves the counter region zero again
-    let ws_len = unsafe { kiln_w4a16_workspace_bytes(m as i32, n as i32, k as i32) };
-    let workspace = Tensor::zeros((ws_len,), DType::U8, a.device())?;
+    // the kernels write every element of the output: no zero fill
+    let out = unsafe { Tensor::empty((m, n), DType::BF16, a.device())? };
+    let workspace = workspace_for(&a, m, n, k)?;
     {
         let (a_s, dev) = device_slice!(a, bf16, "a");
         let (b_s, _) = device_slice!(b_packed, i32, "b_packed");
@@ -76,7 +80,7 @@ pub fn marlin_w4a16_gemm(a: &Tensor, b_packed: &Tensor, scales: &Tensor, groupsi
             let (cp, _g3) = c_s.device_ptr(&stream);
             let (wp, _g4) = w_s.device_ptr(&stream);
             kiln_marlin_w4a16_gemm(ap as *const _, bp as *const _, cp as *mut _, sp as *const _,
-                m as i32, n as i32, k as i32, wp as *mut _, groupsize, 0,
+                m as i32, n as i32, k as i32, wp as *mut _, groupsize, dev.ordinal() as i32,
                 stream.cu_stream() as *mut c_void, -1, -1, -1, 16)
         };
         if status != 0 {
@@ -84,6 +88,31 @@ pub fn marlin_w4a16_gemm(a: &Tensor, b_packed: &Tensor, scales: &Tensor, groupsi
         }
     }
     Ok(out)
+}
+
+/// One workspace per (device ordinal, stream handle).  `kiln_w4a16_workspace_bytes` never
+/// decreases with m, so a buffer that served a larger call serves every smaller one; only the
+/// counter prefix has to be zero, once: every call leaves it zero again.  Calls that share a
+/// workspace are ordered on its stream.
+fn workspace_for(a: &Tensor, m: usize, n: usize, k: usize) -> Result<Tensor> {
+    static CACHE: OnceLock<Mutex<HashMap<(usize, usize), Tensor>>> = OnceLock::new();
+    let need = unsafe { kiln_w4a16_workspace_bytes(m as i32, n as i32, k as i32) };
+    let key = {
+        let (_, dev) = device_slice!(a, bf16, "a");
+        (dev.ordinal(), dev.cuda_stream().cu_stream() as usize)
+    };
+    let mut cache = CACHE.get_or_init(|| Mutex::new(HashMap::new())).lock().unwrap();
+    if let Some(ws) = cache.get(&key) {
+        if ws.elem_count() >= need { return Ok(ws.clone()); }
+    }
+    let zeroed = unsafe { kiln_w4a16_workspace_zeroed_bytes() };
+    let head = Tensor::zeros((zeroed,), DType::U8, a.device())?;
+    let ws = if need > zeroed {
+        let tail = unsafe { Tensor::empty((need - zeroed,), DType::U8, a.device())? };
+        Tensor::cat(&[&head, &tail], 0)?
+    } else { head };
+    cache.insert(key, ws.clone());
+    Ok(ws)
 }
 
 pub mod pack {

@@ -14,6 +14,8 @@ LIB_PATH = Path(__file__).resolve().parent / "lib" / "libkiln_marlin_gemm.so"
 EXPORTS = (
     "kiln_marlin_w4a16_gemm",
     "kiln_w4a16_workspace_bytes",
+    "kiln_w4a16_workspace_bytes_tuned",
+    "kiln_w4a16_workspace_zeroed_bytes",
     "kiln_w4a16_gemm_lora",
     "kiln_w4a16_gemm_swiglu",
     "kiln_w4a16_swiglu_workspace_bytes",
@@ -53,7 +55,19 @@ PROJ_OK, PROJ_SKIPPED, PROJ_ERR = 0, 1, -1
 
 OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_LAUNCH, ERR_ARGUMENT, ERR_ZERO_POINT = range(6)
 
-_lib = None
+# The tuning build: the same sources with -DKILN_W4A16_TUNING_HOOKS, which adds process-wide
+# overrides of the automatic plan (kiln_w4a16_debug_*).  Tests and profiling scripts that pin a
+# kernel instance load it; the shipped library has no such state.
+TUNING_LIB_PATH = LIB_PATH.with_name("libkiln_marlin_gemm_tuning.so")
+
+TUNING_EXPORTS = (
+    "kiln_w4a16_debug_prefill_min_m", "kiln_w4a16_debug_prefill_ks", "kiln_w4a16_debug_prefill_bn",
+    "kiln_w4a16_debug_prefill_bm", "kiln_w4a16_debug_prefill_nb_full", "kiln_w4a16_debug_decode_direct_max_m",
+    "kiln_w4a16_debug_decode_group_major", "kiln_w4a16_debug_decode_runs_per_launch", "kiln_w4a16_debug_tune",
+)
+
+_libs: dict[bool, ctypes.CDLL] = {}
+_active_tuning = False
 
 
 class LibraryMissing(RuntimeError):
@@ -61,20 +75,64 @@ class LibraryMissing(RuntimeError):
 
 
 def load() -> ctypes.CDLL:
-    global _lib
-    if _lib is not None:
-        return _lib
-    if not LIB_PATH.exists():
+    """The library the wrappers call: the shipped one unless `load_tuning()` made the tuning build active."""
+    return _load(_active_tuning)
+
+
+def load_tuning() -> ctypes.CDLL:
+    """Load the tuning build and make it the library the wrappers call until `use_shipped()`."""
+    global _active_tuning
+    L = _load(True)
+    _active_tuning = True
+    return L
+
+
+def use_shipped() -> None:
+    """Back to the shipped library, with every override of the tuning build reset."""
+    global _active_tuning
+    if _active_tuning:
+        L = _libs[True]
+        L.kiln_w4a16_debug_tune(0, 0, 0)
+        L.kiln_w4a16_debug_prefill_min_m(0)
+        L.kiln_w4a16_debug_prefill_ks(0)
+        L.kiln_w4a16_debug_prefill_bn(0)
+        L.kiln_w4a16_debug_prefill_bm(0)
+        L.kiln_w4a16_debug_prefill_nb_full(-1)
+        L.kiln_w4a16_debug_decode_direct_max_m(-1)
+        L.kiln_w4a16_debug_decode_group_major(-1)
+        L.kiln_w4a16_debug_decode_runs_per_launch(0)
+    _active_tuning = False
+
+
+def _load(tuning: bool) -> ctypes.CDLL:
+    if tuning in _libs:
+        return _libs[tuning]
+    path = TUNING_LIB_PATH if tuning else LIB_PATH
+    if not path.exists():
         raise LibraryMissing(
-            f"kiln-marlin-gemm: {LIB_PATH} is not built; run `python -m kiln_amd.build` "
+            f"kiln-marlin-gemm: {path} is not built; run `python -m kiln_amd.build` "
             "(needs hipcc). There is no fallback path.")
-    L = ctypes.CDLL(str(LIB_PATH))
+    L = ctypes.CDLL(str(path))
+    if tuning:
+        for name in TUNING_EXPORTS:
+            fn = getattr(L, name)
+            fn.restype = None
+            fn.argtypes = [ctypes.c_int] * (3 if name == "kiln_w4a16_debug_tune" else 1)
+
     c = ctypes
     vp, i = c.c_void_p, c.c_int
     L.kiln_marlin_w4a16_gemm.restype = i
     L.kiln_marlin_w4a16_gemm.argtypes = [vp, vp, vp, vp, i, i, i, vp, i, i, vp, i, i, i, i]
     L.kiln_w4a16_workspace_bytes.restype = c.c_size_t
     L.kiln_w4a16_workspace_bytes.argtypes = [i, i, i]
+    L.kiln_w4a16_workspace_bytes_tuned.restype = c.c_size_t
+    L.kiln_w4a16_workspace_bytes_tuned.argtypes = [i, i, i, i, i, i]
+    L.kiln_w4a16_workspace_zeroed_bytes.restype = c.c_size_t
+    L.kiln_w4a16_workspace_zeroed_bytes.argtypes = []
+    L.kiln_w4a16_debug_decode_plan.restype = i
+    L.kiln_w4a16_debug_decode_plan.argtypes = [i, i, i, i, c.POINTER(c.c_int)]
+    L.kiln_w4a16_debug_gemm_plan.restype = i
+    L.kiln_w4a16_debug_gemm_plan.argtypes = [i, i, i, i, c.POINTER(c.c_int)]
     L.kiln_w4a16_gemm_lora.restype = i
     L.kiln_w4a16_gemm_lora.argtypes = [vp, vp, vp, vp, i, i, i, vp, i, i, vp, vp, vp, i, i,
                                        c.POINTER(c.c_int), c.POINTER(c.c_float)]
@@ -131,7 +189,7 @@ def load() -> ctypes.CDLL:
     L.kiln_marlin_proj_save.argtypes = [vp, c.c_char_p]
     L.kiln_marlin_proj_load.restype = i
     L.kiln_marlin_proj_load.argtypes = [c.c_char_p, i, pp]
-    _lib = L
+    _libs[tuning] = L
     return L
 
 

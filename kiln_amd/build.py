@@ -14,6 +14,8 @@ from pathlib import Path
 
 CSRC = Path(__file__).resolve().parent / "csrc"
 LIB = Path(__file__).resolve().parent / "lib" / "libkiln_marlin_gemm.so"
+# the same sources with the plan overrides of the test suite compiled in
+TUNING_LIB = LIB.with_name("libkiln_marlin_gemm_tuning.so")
 
 
 def build(force: bool = True, jobs: int = 8, verbose: bool = False) -> Path:
@@ -27,7 +29,7 @@ def build(force: bool = True, jobs: int = 8, verbose: bool = False) -> Path:
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if verbose or res.returncode != 0:
         sys.stderr.write(res.stdout)
-    if res.returncode != 0 or not LIB.exists():
+    if res.returncode != 0 or not LIB.exists() or not TUNING_LIB.exists():
         raise RuntimeError("kiln-marlin-gemm: hipcc build failed")
     return LIB
 

@@ -17,8 +17,8 @@ struct DecodeArgs {
     int *counters;      // N/16 arrival counters, zero on entry and on exit
     int M, N, K, Gs;
     int rows = 0;       // > M (register-fragment instance, M == 32 only): the launch covers `rows` rows of A and
-                        // C, 33...64, in two runs of 32 (grid z), run z with counters + z * N/16 and partial
-                        // tiles + z * KS * 2 * N/16 * 256
+                        // C, 33...128, in up to four runs of 32 (grid z), run z with counters + z * N/16 and
+                        // partial tiles + z * KS * 2 * N/16 * 256
     int KS;             // K slices
     int GS;             // 128-row groups per slice (the last slice may be smaller)
     int U;              // chunks per wavefront, 1..decode_max_run(), <= smallest slice
@@ -75,7 +75,7 @@ struct PrefillArgs {
     // optional fused LoRA epilogue (r_total == 0: none)
     const void *lora_a = nullptr;   // bf16 [r_total, K], adapters stacked along rows
     const void *lora_b = nullptr;   // bf16 [N, r_total], adapters stacked along columns
-    void *lora_t = nullptr;         // prefill_lora_t_bytes(M) bytes of scratch
+    void *lora_t = nullptr;         // prefill_lora_t_bytes(M, few_rows) bytes of scratch
     int r_total = 0;                // <= 64
     int n_adapters = 0;             // <= 8
     const int *ranks = nullptr;     // host arrays of length n_adapters
@@ -92,7 +92,7 @@ struct PrefillArgs {
 };
 
 size_t prefill_aext_bytes(int m, int k);
-size_t prefill_lora_t_bytes(int m);
+size_t prefill_lora_t_bytes(int m, bool few_rows);  // scratch of the LoRA projection on either path
 int prefill_lora_max_slices(int m);
 struct PrefillPlan {
     int bn = 128;     // block columns

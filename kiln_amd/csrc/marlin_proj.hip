@@ -10,6 +10,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
 #include <memory>
 #include <optional>
 #include <string>
@@ -283,7 +284,10 @@ int read_header(std::FILE *f, const char *path, ArtifactHeader &h) {
     if ((int)h.layout_version != kiln_w4a16_layout_version())
         return fail("marlin_proj: artefact layout version " + std::to_string(h.layout_version) + " != library's " +
                     std::to_string(kiln_w4a16_layout_version()) + ": repack " + path);
-    if (!(h.groupsize == -1 || h.groupsize == 128) || !shape_is_supported((int64_t)h.k, (int64_t)h.n) ||
+    // k and n are bounded before they are multiplied: a crafted header must not wrap the products
+    constexpr uint64_t kMaxDim = 1ull << 30;
+    if (!(h.groupsize == -1 || h.groupsize == 128) || h.k > kMaxDim || h.n > kMaxDim ||
+        !shape_is_supported((int64_t)h.k, (int64_t)h.n) ||
         h.b_bytes != h.k * h.n / 2 || h.s_bytes != num_groups((int64_t)h.k, h.groupsize) * h.n * 2)
         return fail(std::string("marlin_proj: inconsistent artefact header: ") + path);
     return KILN_PROJ_OK;
@@ -363,8 +367,12 @@ int load(const char *path, int dev, kiln_marlin_packed_proj_t **out) {
     p.k = k;
     p.n = n;
     p.groupsize = groupsize;
-    p.b_packed_vec.resize((size_t)k * n / 8);
-    p.scales_vec.resize(num_groups(k, groupsize) * (size_t)n);
+    try {  // no exception may cross the C boundary
+        p.b_packed_vec.resize((size_t)k * n / 8);
+        p.scales_vec.resize(num_groups(k, groupsize) * (size_t)n);
+    } catch (const std::exception &) {
+        return fail(std::string("marlin_proj: out of host memory reading ") + path);
+    }
     st = artifact_read(path, p.b_packed_vec.data(), p.scales_vec.data());
     if (st != KILN_PROJ_OK) return st;
     return upload_packed(p, dev, out);

@@ -1,6 +1,8 @@
 // extern "C" entry points of libkiln_marlin_gemm (device side) and the
 // dispatcher that replaces `marlin_cuda` (crates/kiln-marlin-gemm/csrc/marlin_kernel.cu:731-819).
+#include <initializer_list>
 #include <mutex>
+#include <unordered_map>
 
 #include "../../include/kiln_w4a16.h"
 #include "device_common.h"
@@ -46,31 +48,38 @@ struct DecodePlan {
 enum class DecodeMode { kStaged, kDirect, kRegs };
 
 constexpr int kMaxKSlices = 8;  // bounds the partial-tile workspace
-constexpr int kPrefillMinM = 33;  // rows from which the matrix-core prefill kernel takes over
-int g_prefill_min_m = kPrefillMinM;
-bool g_prefill_min_m_forced = false;
-
 constexpr int kDecodeDirectMaxM = 4;  // rows up to which the decode kernel skips the LDS staging of A
-int g_decode_direct_max_m = -1;      // tuning override (-1 = automatic)
-int g_decode_group_major = -1;       // tuning override (0 = never, -1 = where the plan allows)
-int g_decode_runs_per_launch = 0;    // tuning override (1 = one run of rows per launch, 0 = automatic)
-int g_prefill_ks = 0, g_prefill_bn = 0, g_prefill_bm = 0, g_prefill_nb_full = -1;  // tuning overrides (0 / -1 = automatic)
+
+// Overrides of the automatic plan (0 / -1 = automatic).  The shipped library has none: the struct
+// is a compile-time constant there and the entry points have no mutable state besides the plan
+// cache below.  A second build of this file with -DKILN_W4A16_TUNING_HOOKS (the library the test
+// suite and the profiling scripts load for this) makes it a process-wide variable with setters.
+struct Tuning {
+    int prefill_min_m = 0;            // > 0: the matrix-core kernel takes every GEMM of at least this many rows
+    int decode_direct_max_m = -1;
+    int decode_group_major = -1;      // 0 = never, 1 = LDS-staged only, 2 = register-fragment wherever it fits
+    int decode_runs_per_launch = 0;   // 1 = one run of rows per launch
+    int prefill_ks = 0, prefill_bn = 0, prefill_bm = 0, prefill_nb_full = -1;
+    int force_ks = 0, force_u = 0, force_waves = 0;
+};
+#ifdef KILN_W4A16_TUNING_HOOKS
+Tuning g_tune;
+#else
+constexpr Tuning g_tune{};
+#endif
 
 // block shape, whole-tile part and slice count the workspace is sized for and the launch starts from
-PrefillPlan planned_prefill(int m, int n, int k) {
-    PrefillPlan p = plan_prefill(m, n, k, 256, g_prefill_bn, g_prefill_bm);
-    if (g_prefill_nb_full >= 0) p.nb_full = g_prefill_nb_full < n / p.bn ? g_prefill_nb_full : n / p.bn;
-    if (g_prefill_ks > 0) {
-        const int G = k / kGroupK, ks = g_prefill_ks < G ? g_prefill_ks : G, gsb = (G + ks - 1) / ks;
+PrefillPlan planned_prefill(int m, int n, int k, int cus) {
+    PrefillPlan p = plan_prefill(m, n, k, cus, g_tune.prefill_bn, g_tune.prefill_bm);
+    if (g_tune.prefill_nb_full >= 0) p.nb_full = g_tune.prefill_nb_full < n / p.bn ? g_tune.prefill_nb_full : n / p.bn;
+    if (g_tune.prefill_ks > 0) {
+        const int G = k / kGroupK, ks = g_tune.prefill_ks < G ? g_tune.prefill_ks : G, gsb = (G + ks - 1) / ks;
         p.ks = (G + gsb - 1) / gsb;
     }
     // one arrival counter per sliced tile lives in the counter region
     if ((size_t)((m + p.bm - 1) / p.bm) * (n / p.bn - p.nb_full) * sizeof(int) > kCounterBytes) p.ks = 1;
     return p;
 }
-
-// Tuning overrides for experiments (0 = automatic).
-int g_force_ks = 0, g_force_u = 0, g_force_waves = 0;
 
 int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
@@ -106,12 +115,12 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
     const int G = k / kGroupK, NT = n / kTileN;
     int forced_gs = 0;
     if (thread_k > 0) forced_gs = thread_k / kGroupK < G ? thread_k / kGroupK : G;
-    if (g_force_ks) forced_gs = ceil_div(G, g_force_ks);
+    if (g_tune.force_ks) forced_gs = ceil_div(G, g_tune.force_ks);
 
     static const int kWaveOrder[] = {12, 8, 16, 10, 11, 13, 14, 15, 9, 7, 6, 5, 4};
     long best_cost = -1;
     for (int waves : kWaveOrder) {
-        if (g_force_waves ? waves != g_force_waves : waves < 8) continue;
+        if (g_tune.force_waves ? waves != g_tune.force_waves : waves < 8) continue;
         int gs_cap = (decode_max_lds_bytes() - waves * 2048) / (16 * 256) - 1;
         gs_cap = (direct || regs) ? G : (gs_cap < 32 ? gs_cap : 32);
         for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
@@ -124,8 +133,8 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
             if (KS > kMaxKSlices) continue;
             const int u_max = gs_last < decode_max_run() ? gs_last : decode_max_run();
             for (int U = ceil_div(GS, waves); U <= u_max; ++U) {
-                if (g_force_u && U != g_force_u) continue;
-                if (thread_n > 0 && !g_force_u) {  // columns per block -> chunks per block
+                if (g_tune.force_u && U != g_tune.force_u) continue;
+                if (thread_n > 0 && !g_tune.force_u) {  // columns per block -> chunks per block
                     int want = ceil_div((thread_n / kTileN) * GS, waves);
                     want = want < ceil_div(GS, waves) ? ceil_div(GS, waves) : (want > u_max ? u_max : want);
                     if (U != want) continue;
@@ -147,7 +156,7 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
                 probe.U = U;
                 probe.waves = waves;
                 probe.direct = direct;
-                probe.group_major = g_decode_group_major;
+                probe.group_major = g_tune.decode_group_major;
                 if (regs) {
                     if (!decode_group_major_regs_ok(probe)) continue;
                     cost -= gm_gain;
@@ -161,7 +170,7 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
             // wavefronts as evenly as they go (12 wavefronts take 20 groups as 8 x 2 + 4 x 1)
             for (int T = 2; T <= 6 && mode == DecodeMode::kStaged && rows <= 16 && thread_n <= 0; ++T) {
                 const int U = T * ceil_div(GS, waves);
-                if (U > decode_max_run() || (g_force_u && U != g_force_u)) continue;
+                if (U > decode_max_run() || (g_tune.force_u && U != g_tune.force_u)) continue;
                 DecodeArgs probe;
                 probe.M = rows;
                 probe.K = k;
@@ -170,7 +179,7 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
                 probe.U = U;
                 probe.waves = waves;
                 probe.gm_tiles = T;
-                probe.group_major = g_decode_group_major;
+                probe.group_major = g_tune.decode_group_major;
                 if (!decode_group_major_ok(probe)) continue;
                 const int BPS = ceil_div(NT, T);
                 const int rounds = ceil_div(BPS * KS, cus);
@@ -195,16 +204,16 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
 constexpr long kRegsHandicap = 8;
 bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, DecodePlan *plan, bool *direct) {
     *direct = false;
-    const bool regs_allowed = g_decode_group_major != 0 && g_decode_group_major != 1 && thread_n <= 0;
+    const bool regs_allowed = g_tune.decode_group_major != 0 && g_tune.decode_group_major != 1 && thread_n <= 0;
     if (m > 16) return regs_allowed && plan_decode(n, k, cus, thread_k, thread_n, DecodeMode::kRegs, m, plan);
-    if (g_decode_direct_max_m >= 0 && m <= g_decode_direct_max_m) {  // tuning override
+    if (g_tune.decode_direct_max_m >= 0 && m <= g_tune.decode_direct_max_m) {  // tuning override
         *direct = true;
         return plan_decode(n, k, cus, thread_k, thread_n, DecodeMode::kDirect, m, plan);
     }
     const bool have_staged = plan_decode(n, k, cus, thread_k, thread_n, DecodeMode::kStaged, m, plan);
     DecodePlan rp;
     if (regs_allowed && plan_decode(n, k, cus, thread_k, thread_n, DecodeMode::kRegs, m, &rp) &&
-        (!have_staged || g_decode_group_major == 2 || rp.cost + kRegsHandicap < plan->cost ||
+        (!have_staged || g_tune.decode_group_major == 2 || rp.cost + kRegsHandicap < plan->cost ||
          // few rows, one or two chunks per wavefront: no staging and no barrier wins (cfg 0: 3.4 against 3.8 us)
          (m <= kDecodeDirectMaxM && rp.U <= 2 && rp.cost <= plan->cost))) {
         *plan = rp;
@@ -213,39 +222,185 @@ bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, Dec
     if (!have_staged) return false;
     // few rows and short runs: latency-bound launches, where skipping the staging barrier wins
     // (measured: -0.3...-1.0 us at M <= 4 with up to 3 chunks per wavefront, +0.7 us with 6)
-    *direct = g_decode_direct_max_m < 0 && m <= kDecodeDirectMaxM && plan->U <= 3 && plan->gm_tiles == 0;
+    *direct = g_tune.decode_direct_max_m < 0 && m <= kDecodeDirectMaxM && plan->U <= 3 && plan->gm_tiles == 0;
     return true;
 }
 
-// Rows from which the matrix-core kernel runs the plain GEMM.  Below, the rows go through the
-// small-M kernel in slabs, one launch each, every launch streaming the weights again: slabs of
-// 32 rows where the plan fits the two-slab kernel instance, of 16 otherwise.  Measured against
-// the 64-row blocks of the other kernel (16-24 us at any M <= 64): for projections of up to
-// 32 M weights two 32-row launches (2 x 7.9 ... 10.9 us) or three 16-row launches (14.5-16.4 us)
-// still win; the fused gate+up projection changes over at 33 rows.
-// Does a GEMM of m rows take the matrix-core kernel?  Where a plan for the two-slab small-M
-// instance exists, up to 80 rows go there (runs of 32 rows, up to four per launch); measured
-// against the matrix-core kernel's 64-row blocks it is ahead or level up to 80 rows on all four
-// projection shapes (at 72 rows 28.3 / 27.5 / 18.1 / 16.2 us against 32.2 / 27.1 / 18.9 / 18.5)
-// and behind from 96 rows on.  The one exception is the widest projection at 49...64 rows, where
-// one round of 64-row blocks (20.1 us) is ahead of two runs (20.2...21.0).
-bool takes_prefill(int m, int n, int k, int cus) {
-    if (g_prefill_min_m_forced) return m >= g_prefill_min_m;
-    DecodePlan plan;
+// The slab plans are pure functions of (rows, n, k, compute units, overrides) and cost 15-25 us
+// of host time each, more than the GEMM they plan, so they are kept: a small table behind a
+// mutex (the entry points may be entered from several threads at once).
+struct SlabKey {
+    int m, n, k, cus, thread_k, thread_n;
+    bool operator==(const SlabKey &o) const {
+        return m == o.m && n == o.n && k == o.k && cus == o.cus && thread_k == o.thread_k && thread_n == o.thread_n;
+    }
+};
+struct SlabKeyHash {
+    size_t operator()(const SlabKey &key) const {
+        size_t h = 1469598103934665603ull;
+        for (int v : {key.m, key.n, key.k, key.cus, key.thread_k, key.thread_n}) h = (h ^ (size_t)(unsigned)v) * 1099511628211ull;
+        return h;
+    }
+};
+struct SlabChoice {
+    bool ok = false;
     bool direct = false;
-    if (!choose_decode(32, n, k, cus, -1, -1, &plan, &direct)) return m >= 49;
+    DecodePlan plan{};
+};
+std::mutex g_plan_mutex;
+std::unordered_map<SlabKey, SlabChoice, SlabKeyHash> g_plan_cache;
+
+SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n) {
+    const SlabKey key{m, n, k, cus, thread_k, thread_n};
+    {
+        std::lock_guard<std::mutex> lock(g_plan_mutex);
+        auto it = g_plan_cache.find(key);
+        if (it != g_plan_cache.end()) return it->second;
+    }
+    SlabChoice c;
+    c.ok = choose_decode(m, n, k, cus, thread_k, thread_n, &c.plan, &c.direct);
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    if (g_plan_cache.size() > 4096) g_plan_cache.clear();  // a caller cycling through many shapes
+    g_plan_cache.emplace(key, c);
+    return c;
+}
+
+// Does a GEMM of m rows take the matrix-core kernel?  Below the change-over the rows go through
+// the small-M kernels in runs, every launch streaming the weights again.  Where a plan for the
+// two-slab small-M instance exists, up to 80 rows go there (runs of 32 rows, up to four per
+// launch); measured against the matrix-core kernel's 64-row blocks (16-24 us at any M <= 64) it is
+// ahead or level up to 80 rows on all four projection shapes (at 72 rows 28.3 / 27.5 / 18.1 /
+// 16.2 us against 32.2 / 27.1 / 18.9 / 18.5) and behind from 96 rows on.  The one exception is the
+// widest projection at 49...64 rows, where one round of 64-row blocks (20.1 us) is ahead of two
+// runs (20.2...21.0).  Without such a plan the matrix-core kernel starts at 49 rows.
+bool takes_prefill(int m, int n, int k, int cus) {
+    if (g_tune.prefill_min_m > 0) return m >= g_tune.prefill_min_m;
+    if (!slab_choice(32, n, k, cus, -1, -1).ok) return m >= 49;
     if ((long)n * k > (32L << 20) && m >= 49 && m <= 64) return true;
     return m >= 81;
 }
 
-// workspace layout: counters | decode partial tiles | prefill row-sum operands | LoRA projection |
-// prefill partial tiles
-size_t partial_bytes(int n);
-size_t prefill_scratch_offset(int m, int n, int k) {
-    return kCounterBytes + partial_bytes(n) + prefill_aext_bytes(m, k) + prefill_lora_t_bytes(m);
+// Everything the dispatcher decides for one call, as a pure function of the shape, the compute
+// units and the overrides: kiln_w4a16_workspace_bytes and the launch path both start from it, so
+// the workspace is sized for exactly what the call will use.
+constexpr int kMaxDecodeLaunches = 16;
+struct DecodeLaunch {
+    int r0;        // first row
+    int M;         // rows per run (<= 32)
+    int rows;      // > M: the launch covers this many rows in runs of M (grid z)
+    DecodePlan plan;
+    bool direct;
+};
+struct GemmPlan {
+    bool prefill = false;
+    PrefillPlan pf{};
+    int launches = 0;
+    DecodeLaunch dl[kMaxDecodeLaunches];
+    size_t decode_partial = 0;  // bytes of partial tiles the largest launch exchanges
+};
+
+// f32 partial tiles one small-M launch may exchange: per run and K slice two parts of N x 16.
+// Plans of whole tiles in one slice exchange nothing.
+size_t decode_launch_partial_bytes(const DecodeLaunch &l, int n, int k) {
+    const DecodePlan &p = l.plan;
+    bool exchanges = p.KS > 1;
+    if (!p.regs && p.gm_tiles == 0) {  // tile-major runs: blocks may cut tiles
+        const int G = k / kGroupK, gs_last = G - (p.KS - 1) * p.GS, R = p.waves * p.U;
+        exchanges = exchanges || R % p.GS != 0 || R % gs_last != 0;
+    }
+    if (!exchanges) return 0;
+    const int runs = l.rows > l.M ? (l.rows + l.M - 1) / l.M : 1;
+    return (size_t)runs * p.KS * 2 * (size_t)n * 16 * sizeof(float);
 }
 
-size_t partial_bytes(int n) { return (size_t)kMaxKSlices * 2 * (size_t)n * 16 * sizeof(float); }
+void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, GemmPlan *gp) {
+    gp->prefill = true;
+    gp->launches = 0;
+    gp->decode_partial = 0;
+    PrefillPlan p = planned_prefill(m, n, k, cus);
+    if ((thread_n == 128 || thread_n == 256) && thread_n != p.bn) {  // block columns: whole tiles only
+        p.bn = thread_n;
+        p.nb_full = n / thread_n;
+        p.ks = 1;
+    }
+    // thread_k asks for a K slice length; it can lower the slice count but never raise it
+    if (thread_k > 0) {
+        const int G = k / kGroupK, gs = thread_k / kGroupK < G ? thread_k / kGroupK : G;
+        const int want = ceil_div(G, gs);
+        if (want < p.ks) p.ks = want;
+    }
+    gp->pf = p;
+}
+
+void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, GemmPlan *gp) {
+    *gp = GemmPlan{};
+    // the small-M kernels keep one arrival counter per column tile (and run) in the counter region
+    const bool counters_fit = (size_t)(n / kTileN) * sizeof(int) <= kCounterBytes;
+    if (!counters_fit || takes_prefill(m, n, k, cus)) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
+    // Runs of A, one launch each -- launches on one stream run in order, so they may share the
+    // workspace -- of 16 rows, or of up to 32 where the plan fits the kernel instance that takes two
+    // 16-row slabs in one pass over the weights; where more than 32 rows are left and that
+    // instance runs, up to four runs of 32 share one launch (a later run's blocks fill the units the
+    // earlier ones leave idle; each run has its own counters and partial tiles).
+    for (int r0 = 0; r0 < m;) {
+        if (gp->launches == kMaxDecodeLaunches) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
+        DecodeLaunch &l = gp->dl[gp->launches];
+        const int left = m - r0;
+        l.r0 = r0;
+        l.M = left < 32 ? left : 32;
+        SlabChoice c;
+        if (l.M > 16) c = slab_choice(l.M, n, k, cus, thread_k, thread_n);
+        if (!c.ok) {
+            l.M = left < 16 ? left : 16;
+            c = slab_choice(l.M, n, k, cus, thread_k, thread_n);
+            // no small-M plan (K beyond eight slices of 32 groups): the matrix-core kernel takes any M
+            if (!c.ok) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
+        }
+        l.plan = c.plan;
+        l.direct = c.direct;
+        l.rows = 0;
+        int max_runs = kMaxKSlices / l.plan.KS < 4 ? kMaxKSlices / l.plan.KS : 4;
+        if ((size_t)max_runs * (n / kTileN) * sizeof(int) > kCounterBytes) max_runs = 1;
+        if (g_tune.decode_runs_per_launch > 0 && max_runs > g_tune.decode_runs_per_launch)
+            max_runs = g_tune.decode_runs_per_launch;
+        int step = l.M;
+        if (l.M == 32 && l.plan.regs && left > 32 && max_runs >= 2) {
+            l.rows = left < 32 * max_runs ? left : 32 * max_runs;
+            step = l.rows;
+        }
+        const size_t pb = decode_launch_partial_bytes(l, n, k);
+        if (pb > gp->decode_partial) gp->decode_partial = pb;
+        ++gp->launches;
+        r0 += step;
+    }
+}
+
+// workspace of one call: counters | small-M partial tiles | LoRA projection           (small-M path)
+//                        counters | row-sum operands | LoRA projection | partial tiles (matrix-core path)
+struct WorkspaceLayout {
+    size_t decode_partial, aext, lora_t, prefill_partial, total;
+};
+WorkspaceLayout workspace_layout(const GemmPlan &gp, int m, int n, int k) {
+    WorkspaceLayout w{};
+    size_t off = kCounterBytes;
+    if (gp.prefill) {
+        w.aext = off;
+        off += prefill_aext_bytes(m, k);
+        w.lora_t = off;
+        off += prefill_lora_t_bytes(m, false);
+        off = (off + 255) & ~(size_t)255;
+        w.prefill_partial = off;
+        off += prefill_partial_bytes(m, n, gp.pf);
+    } else {
+        w.decode_partial = off;
+        off += gp.decode_partial;
+        off = (off + 255) & ~(size_t)255;
+        w.lora_t = off;
+        off += prefill_lora_t_bytes(m, true);
+    }
+    w.total = off;
+    return w;
+}
 
 __global__ void dequant_f32_kernel(const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
                                    float *__restrict__ out, int K, int N, int Gs) {
@@ -313,6 +468,25 @@ struct LoraSpec {
     const float *scales;
 };
 
+// Bytes a call of m rows needs, made monotone in m: the largest need of any m' <= m.  The plan
+// (and with it the need) changes with m' only through the small-M runs (m' <= 128 here; beyond
+// that only overrides keep a call on that path) and through the matrix-core kernel's row blocks
+// of 64 or 128 rows, so those m' are the ones evaluated.
+size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thread_n) {
+    size_t most = 0;
+    auto consider = [&](int mm) {
+        GemmPlan gp;
+        plan_gemm(mm, n, k, cus, thread_k, thread_n, &gp);
+        const size_t need = workspace_layout(gp, mm, n, k).total;
+        if (need > most) most = need;
+    };
+    const int small = g_tune.prefill_min_m > 128 ? g_tune.prefill_min_m : 128;
+    for (int mm = 1; mm <= m && mm <= small; ++mm) consider(mm);
+    for (int mm = 64; mm < m; mm += 64) consider(mm);
+    consider(m);
+    return most;
+}
+
 // The GEMM behind every entry point: small-M or matrix-core path by row count, with the
 // optional low-rank term.
 kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
@@ -325,17 +499,20 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     if (prob_m == 0 || prob_n == 0 || prob_k == 0) return KILN_W4A16_OK;  // marlin_kernel.cu:772-773
     if (!A || !B || !C || !s || !workspace) return KILN_W4A16_ERR_ARGUMENT;
 
-    char *lora_t = reinterpret_cast<char *>(workspace) + kCounterBytes + partial_bytes(prob_n) +
-                   prefill_aext_bytes(prob_m, prob_k);
     const int cus = sms > 0 ? sms : compute_units(dev);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (takes_prefill(prob_m, prob_n, prob_k, cus)) {
+    GemmPlan gp;
+    plan_gemm(prob_m, prob_n, prob_k, cus, thread_k, thread_n, &gp);
+    const WorkspaceLayout wl = workspace_layout(gp, prob_m, prob_n, prob_k);
+    char *ws = reinterpret_cast<char *>(workspace);
+    char *lora_t = ws + wl.lora_t;
+    if (gp.prefill) {
         PrefillArgs pa{};
         pa.A = A;
         pa.B = B;
         pa.S = s;
         pa.C = C;
-        pa.aext = reinterpret_cast<char *>(workspace) + kCounterBytes + partial_bytes(prob_n);
+        pa.aext = ws + wl.aext;
         pa.M = prob_m;
         pa.N = prob_n;
         pa.K = prob_k;
@@ -349,33 +526,18 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             pa.ranks = lora->ranks;
             pa.scales = lora->scales;
         }
-        // thread_k asks for a K slice length; it can lower the slice count but never
-        // raise it above what kiln_w4a16_workspace_bytes sized the scratch for
         pa.cus = cus;
-        const PrefillPlan plan = planned_prefill(prob_m, prob_n, prob_k);
-        pa.KS = plan.ks;
-        pa.bn = plan.bn;
-        pa.bm = plan.bm;
-        pa.nb_full = plan.nb_full;
-        if ((thread_n == 128 || thread_n == 256) && thread_n != plan.bn) {  // block columns: whole tiles only
-            pa.bn = thread_n;
-            pa.nb_full = prob_n / thread_n;
-            pa.KS = 1;
-        }
-        if (thread_k > 0) {
-            const int G = prob_k / kGroupK, gs = thread_k / kGroupK < G ? thread_k / kGroupK : G;
-            const int want = ceil_div(G, gs);
-            if (want < pa.KS) pa.KS = want;
-        }
+        pa.KS = gp.pf.ks;
+        pa.bn = gp.pf.bn;
+        pa.bm = gp.pf.bm;
+        pa.nb_full = gp.pf.nb_full;
         pa.counters = reinterpret_cast<int *>(workspace);
-        pa.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) +
-                                               prefill_scratch_offset(prob_m, prob_n, prob_k));
+        pa.partial = reinterpret_cast<float *>(ws + wl.prefill_partial);
         return launch_prefill(pa, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
     }
-    if ((size_t)(prob_n / kTileN) * sizeof(int) > kCounterBytes) return KILN_W4A16_ERR_KERN_SHAPE;
 
     int rp = 0, lora_slices = 1;
-    if (lora) {  // the scaled projection of all rows onto the adapters, once, ahead of the slabs
+    if (lora) {  // the scaled projection of all rows onto the adapters, once, ahead of the runs
         PrefillArgs pj{};
         pj.A = A;
         pj.M = prob_m;
@@ -393,53 +555,33 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     a.B = B;
     a.S = s;
     a.counters = reinterpret_cast<int *>(workspace);
-    a.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + kCounterBytes);
+    a.partial = reinterpret_cast<float *>(ws + wl.decode_partial);
     a.N = prob_n;
     a.K = prob_k;
     a.Gs = (groupsize == -1) ? 1 : prob_k / kGroupK;
-    // Slabs of A, one launch each; launches on one stream run in order, so they may share the
-    // workspace.  A slab has 16 rows, or up to 32 where the plan fits the kernel instance that
-    // takes two 16-row slabs in one pass over the weights.
-    for (int r0 = 0; r0 < prob_m; r0 += a.M) {
-        a.A = reinterpret_cast<const uint16_t *>(A) + (size_t)r0 * prob_k;
-        a.C = reinterpret_cast<uint16_t *>(C) + (size_t)r0 * prob_n;
+    for (int i = 0; i < gp.launches; ++i) {
+        const DecodeLaunch &l = gp.dl[i];
+        a.A = reinterpret_cast<const uint16_t *>(A) + (size_t)l.r0 * prob_k;
+        a.C = reinterpret_cast<uint16_t *>(C) + (size_t)l.r0 * prob_n;
         if (lora) {
-            a.lora_t = reinterpret_cast<const uint16_t *>(lora_t) + (size_t)r0 * rp;
+            a.lora_t = reinterpret_cast<const uint16_t *>(lora_t) + (size_t)l.r0 * rp;
             a.lora_b = lora->b;
             a.r_total = lora->r_total;
             a.lora_slices = lora_slices;
             a.lora_rows = prob_m;
         }
-        const int left = prob_m - r0;
-        DecodePlan plan;
-        a.M = left < 32 ? left : 32;
-        if (a.M <= 16 || !choose_decode(a.M, prob_n, prob_k, cus, thread_k, thread_n, &plan, &a.direct)) {
-            a.M = left < 16 ? left : 16;
-            if (!choose_decode(a.M, prob_n, prob_k, cus, thread_k, thread_n, &plan, &a.direct))
-                return KILN_W4A16_ERR_KERN_SHAPE;
-        }
-        a.KS = plan.KS;
-        a.GS = plan.GS;
-        a.U = plan.U;
-        a.BPS = plan.BPS;
-        a.waves = plan.waves;
-        a.regs = plan.regs;
-        a.gm_tiles = plan.gm_tiles;
-        a.group_major = g_decode_group_major;
-        // two runs of up to 32 rows in one launch (the second run through the same two-slab kernel
-        // instance even if one slab would do: a second launch costs more than the idle slab) where
-        // the workspace holds two sets of partial tiles
-        a.rows = 0;
-        int step = a.M;
-        int max_runs = kMaxKSlices / a.KS < 4 ? kMaxKSlices / a.KS : 4;
-        if ((size_t)max_runs * (prob_n / kTileN) * sizeof(int) > kCounterBytes) max_runs = 1;
-        if (g_decode_runs_per_launch > 0 && max_runs > g_decode_runs_per_launch) max_runs = g_decode_runs_per_launch;
-        if (a.M == 32 && a.regs && left > 32 && max_runs >= 2) {
-            a.rows = left < 32 * max_runs ? left : 32 * max_runs;
-            step = a.rows;
-        }
+        a.M = l.M;
+        a.rows = l.rows;
+        a.direct = l.direct;
+        a.KS = l.plan.KS;
+        a.GS = l.plan.GS;
+        a.U = l.plan.U;
+        a.BPS = l.plan.BPS;
+        a.waves = l.plan.waves;
+        a.regs = l.plan.regs;
+        a.gm_tiles = l.plan.gm_tiles;
+        a.group_major = g_tune.decode_group_major;
         if (launch_decode(a, st) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
-        r0 += step - a.M;  // the loop adds a.M
     }
     return KILN_W4A16_OK;
 }
@@ -450,14 +592,19 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
 extern "C" {
 
 size_t kiln_w4a16_workspace_bytes(int prob_m, int prob_n, int prob_k) {
-    if (prob_n <= 0 || prob_k <= 0) return kCounterBytes;
-    // worst case over the plans the dispatcher may pick: K split down to one
-    // group per wavefront
-    // counters | partial tiles | prefill row-sum operands | LoRA projection (both paths use it)
-    const int m = prob_m > 0 ? prob_m : 1;
-    return prefill_scratch_offset(m, prob_n, prob_k) +
-           prefill_partial_bytes(m, prob_n, planned_prefill(m, prob_n, prob_k));
+    return kiln_w4a16_workspace_bytes_tuned(prob_m, prob_n, prob_k, -1, -1, -1);
 }
+
+size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k, int thread_k, int thread_n, int sms) {
+    if (prob_n <= 0 || prob_k <= 0 || !shape_ok(prob_n, prob_k, 128)) return kCounterBytes;
+    int dev = 0;
+    if (sms <= 0 && hipGetDevice(&dev) != hipSuccess) dev = -1;  // no device: the part's 256 units
+    const int cus = sms > 0 ? sms : compute_units(dev);
+    return workspace_bytes_upto(prob_m > 0 ? prob_m : 1, prob_n, prob_k, cus, thread_k > 0 ? thread_k : -1,
+                                thread_n > 0 ? thread_n : -1);
+}
+
+size_t kiln_w4a16_workspace_zeroed_bytes(void) { return kCounterBytes; }
 
 kiln_marlin_status_t kiln_marlin_w4a16_gemm(const void *A, const void *B, void *C, void *s,
                                             int prob_m, int prob_n, int prob_k, void *workspace,
@@ -468,41 +615,55 @@ kiln_marlin_status_t kiln_marlin_w4a16_gemm(const void *A, const void *B, void *
                     nullptr);
 }
 
-// Not part of the public header: process-wide overrides of the automatic plan for profiling
-// scripts and the block-shape tests (0 / -1 = automatic).  Plain globals: set them only while no
-// other thread is inside a GEMM call.
-void kiln_w4a16_debug_prefill_min_m(int m) {
-    g_prefill_min_m = m > 0 ? m : kPrefillMinM;
-    g_prefill_min_m_forced = m > 0;
-}
-void kiln_w4a16_debug_prefill_ks(int ks) { g_prefill_ks = ks; }
-void kiln_w4a16_debug_prefill_bn(int bn) { g_prefill_bn = bn; }
-void kiln_w4a16_debug_decode_direct_max_m(int m) { g_decode_direct_max_m = m; }
-void kiln_w4a16_debug_prefill_bm(int bm) { g_prefill_bm = bm; }
-void kiln_w4a16_debug_prefill_nb_full(int nb) { g_prefill_nb_full = nb; }
-
-// The decode plan for a slab of m rows on a part with `cus` compute units (no GPU needed):
-// out = {KS, GS, U, BPS, waves, direct, regs, gm_tiles}.  m <= 32; returns 0, or 1 if no plan fits.
+// The small-M plan for a run of m rows on a part with `cus` compute units (a pure query, no GPU
+// needed; not part of the public header): out = {KS, GS, U, BPS, waves, direct, regs, gm_tiles}.
+// m <= 32; returns 0, or 1 if no plan fits.
 int kiln_w4a16_debug_decode_plan(int m, int n, int k, int cus, int *out) {
-    DecodePlan p;
-    bool direct = false;
-    if (m < 1 || m > 32 || cus < 1 || !shape_ok(n, k, 128) || !choose_decode(m, n, k, cus, -1, -1, &p, &direct))
-        return 1;
+    if (m < 1 || m > 32 || cus < 1 || !shape_ok(n, k, 128)) return 1;
+    const SlabChoice c = slab_choice(m, n, k, cus, -1, -1);
+    if (!c.ok) return 1;
+    const DecodePlan &p = c.plan;
     out[0] = p.KS; out[1] = p.GS; out[2] = p.U; out[3] = p.BPS; out[4] = p.waves;
-    out[5] = direct;
+    out[5] = c.direct;
     out[6] = p.regs;
     out[7] = p.gm_tiles;
     return 0;
 }
 
-void kiln_w4a16_debug_decode_group_major(int mode) { g_decode_group_major = mode; }
-void kiln_w4a16_debug_decode_runs_per_launch(int runs) { g_decode_runs_per_launch = runs; }
-
-void kiln_w4a16_debug_tune(int waves, int run, int kslices) {
-    g_force_waves = waves;
-    g_force_u = run;
-    g_force_ks = kslices;
+// Which path a plain GEMM takes (a pure query, not part of the public header):
+// out = {matrix-core path?, launches, block rows, block columns, whole column blocks, K slices}.
+int kiln_w4a16_debug_gemm_plan(int m, int n, int k, int cus, int *out) {
+    if (m < 1 || cus < 1 || !shape_ok(n, k, 128)) return 1;
+    GemmPlan gp;
+    plan_gemm(m, n, k, cus, -1, -1, &gp);
+    out[0] = gp.prefill; out[1] = gp.launches; out[2] = gp.pf.bm; out[3] = gp.pf.bn; out[4] = gp.pf.nb_full;
+    out[5] = gp.pf.ks;
+    return 0;
 }
+
+#ifdef KILN_W4A16_TUNING_HOOKS
+// Only in the tuning build of the library (never in the shipped one): process-wide overrides of
+// the automatic plan for the test suite and profiling scripts (0 / -1 = automatic).  Plain
+// globals: set them only while no other thread is inside a GEMM call.
+static void tuning_changed() {
+    std::lock_guard<std::mutex> lock(g_plan_mutex);
+    g_plan_cache.clear();
+}
+void kiln_w4a16_debug_prefill_min_m(int m) { g_tune.prefill_min_m = m > 0 ? m : 0; tuning_changed(); }
+void kiln_w4a16_debug_prefill_ks(int ks) { g_tune.prefill_ks = ks; }
+void kiln_w4a16_debug_prefill_bn(int bn) { g_tune.prefill_bn = bn; }
+void kiln_w4a16_debug_prefill_bm(int bm) { g_tune.prefill_bm = bm; }
+void kiln_w4a16_debug_prefill_nb_full(int nb) { g_tune.prefill_nb_full = nb; }
+void kiln_w4a16_debug_decode_direct_max_m(int m) { g_tune.decode_direct_max_m = m; tuning_changed(); }
+void kiln_w4a16_debug_decode_group_major(int mode) { g_tune.decode_group_major = mode; tuning_changed(); }
+void kiln_w4a16_debug_decode_runs_per_launch(int runs) { g_tune.decode_runs_per_launch = runs; }
+void kiln_w4a16_debug_tune(int waves, int run, int kslices) {
+    g_tune.force_waves = waves;
+    g_tune.force_u = run;
+    g_tune.force_ks = kslices;
+    tuning_changed();
+}
+#endif
 
 kiln_marlin_status_t kiln_w4a16_dequant_f32(const void *B, const void *s, int prob_k, int prob_n,
                                             int groupsize, void *out, int dev, void *stream) {
@@ -523,7 +684,6 @@ kiln_marlin_status_t kiln_w4a16_gemm_lora(const void *A, const void *B, void *C,
                                           int groupsize, int dev, void *stream, const void *lora_a,
                                           const void *lora_b, int r_total, int n_adapters,
                                           const int *ranks, const float *scales) {
-    (void)dev;
     if (prob_m < 0 || prob_n < 0 || prob_k < 0) return KILN_W4A16_ERR_PROB_SHAPE;
     if (!shape_ok(prob_n, prob_k, groupsize)) return KILN_W4A16_ERR_PROB_SHAPE;
     if (r_total < 1 || n_adapters < 1 || !ranks || !scales) return KILN_W4A16_ERR_ARGUMENT;
@@ -554,7 +714,8 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu(const void *A, const void *B, void *
     if (prob_m == 0 || n_out == 0 || prob_k == 0) return KILN_W4A16_OK;
     if (!A || !B || !C || !s || !workspace) return KILN_W4A16_ERR_ARGUMENT;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    if (prob_m < g_prefill_min_m && prob_m <= 32) {
+    const int cus = compute_units(dev);
+    if (prob_m <= 32 && !(g_tune.prefill_min_m > 0 && prob_m >= g_tune.prefill_min_m)) {
         // decode regime: the GEMM as usual into scratch behind the workspace, then one
         // elementwise pass over the few rows
         uint16_t *tmp = reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(workspace) +
@@ -567,33 +728,46 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu(const void *A, const void *B, void *
         swiglu_rows_kernel<<<(items + 255) / 256, 256, 0, st>>>(tmp, reinterpret_cast<uint16_t *>(C), prob_m, n_out);
         return hipGetLastError() == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
     }
+    GemmPlan gp;
+    plan_as_prefill(prob_m, prob_n, prob_k, cus, -1, -1, &gp);
+    const WorkspaceLayout wl = workspace_layout(gp, prob_m, prob_n, prob_k);
     PrefillArgs pa{};
     pa.A = A;
     pa.B = B;
     pa.S = s;
     pa.C = C;
-    pa.aext = reinterpret_cast<char *>(workspace) + kCounterBytes + partial_bytes(prob_n);
+    pa.aext = reinterpret_cast<char *>(workspace) + wl.aext;
     pa.M = prob_m;
     pa.N = prob_n;
     pa.K = prob_k;
     pa.Gs = (groupsize == -1) ? 1 : prob_k / kGroupK;
     pa.swiglu = true;
-    pa.cus = compute_units(dev);
-    const PrefillPlan plan = planned_prefill(prob_m, prob_n, prob_k);
-    pa.KS = plan.ks;
-    pa.bn = plan.bn;
-    pa.bm = plan.bm;
-    pa.nb_full = plan.nb_full;
+    pa.cus = cus;
+    pa.KS = gp.pf.ks;
+    pa.bn = gp.pf.bn;
+    pa.bm = gp.pf.bm;
+    pa.nb_full = gp.pf.nb_full;
     pa.counters = reinterpret_cast<int *>(workspace);
-    pa.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) +
-                                           prefill_scratch_offset(prob_m, prob_n, prob_k));
+    pa.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + wl.prefill_partial);
     return launch_prefill(pa, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
 }
 
 size_t kiln_w4a16_swiglu_workspace_bytes(int prob_m, int n_out, int prob_k) {
     const int m = prob_m > 0 ? prob_m : 1;
-    // the GEMM's own workspace, then room for the decode regime's [32, 2 n_out] bf16 intermediate
-    return swiglu_tmp_offset(m, 2 * n_out, prob_k) + (size_t)32 * 2 * n_out * sizeof(uint16_t);
+    if (n_out <= 0 || prob_k <= 0 || !shape_ok(2 * n_out, prob_k, 128)) return kCounterBytes;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = -1;
+    const int cus = compute_units(dev);
+    // the plain GEMM's need for every m' <= m (rows up to 32 run it), the matrix-core path's need for
+    // every row-block count up to m's, and room for the decode regime's [32, 2 n_out] bf16 intermediate
+    size_t most = swiglu_tmp_offset(m, 2 * n_out, prob_k) + (size_t)32 * 2 * n_out * sizeof(uint16_t);
+    for (int mm = 64; mm < m + 64; mm += 64) {
+        GemmPlan gp;
+        plan_as_prefill(mm < m ? mm : m, 2 * n_out, prob_k, cus, -1, -1, &gp);
+        const size_t need = workspace_layout(gp, mm < m ? mm : m, 2 * n_out, prob_k).total;
+        if (need > most) most = need;
+    }
+    return most;
 }
 
 }  // extern "C"

@@ -434,9 +434,12 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_decode_kernel(
     if (KS == 1 && blk0 == tf * gs && blk1 == (tl + 1) * gs) return;  // nothing was exchanged
 
     // Exchange of partial tiles.  They are written and read with device-scope
-    // atomic accesses (no whole-cache write-back or invalidate); the barrier
-    // waits for this block's stores before its arrivals are counted.  For each
-    // tile, the last contributor to arrive adds all parts in ascending K order.
+    // atomic accesses (no whole-cache write-back or invalidate).  A barrier by itself
+    // orders nothing outside the workgroup, so every wavefront first waits until its own
+    // stores have been acknowledged (vmcnt(0)); only then does the barrier let the block's
+    // arrivals be counted.  For each tile, the last contributor to arrive adds all parts
+    // in ascending K order.
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
     if (tid < ntouched) {
         const int tt = tf + tid;
@@ -617,7 +620,9 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_decode_gm_kernel(
     }
     if (KS == 1) return;
 
-    // exchange between the slices: as in the kernel above, one part per slice
+    // exchange between the slices: as in the kernel above, one part per slice (every
+    // wavefront's stores acknowledged, then the barrier, then the arrival is counted)
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
     if (tid < tiles)
         s_last[tid] = __hip_atomic_fetch_add(counters + tf + tid, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KS - 1;
@@ -825,7 +830,9 @@ __global__ __launch_bounds__(12 * 64) void w4a16_decode_gmr_kernel(
     }
     if (KS == 1) return;
 
-    // exchange between the slices: one part per slice and slab
+    // exchange between the slices: one part per slice and slab (every wavefront's stores
+    // acknowledged, then the barrier, then the arrival is counted)
+    __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
     __syncthreads();
     if (tid < tiles) {
         const bool last =

@@ -214,7 +214,10 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
                     __hip_atomic_store(tile0 + ((size_t)(blockIdx.y * (IT * 4) + item) * 4 + i) * 64, acc[it][i],
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __syncthreads();  // waits for this block's stores before its arrival is counted
+        // each wavefront waits until its own stores have been acknowledged (a barrier alone
+        // orders nothing outside the workgroup); after the barrier the arrival is counted
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
         if (tid == 0)
             s_last = __hip_atomic_fetch_add(counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KZ - 1;
         __syncthreads();
@@ -751,7 +754,10 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
                 for (int r = 0; r < 16; ++r)
                     __hip_atomic_store(mine + ((mi * 2 + ni) * 16 + r) * NT + tid, acc[mi][ni][r],
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        __syncthreads();  // waits for this block's stores before its arrival is counted
+        // each wavefront waits until its own stores have been acknowledged (a barrier alone
+        // orders nothing outside the workgroup); after the barrier the arrival is counted
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
         KILN_TL(3);
         if (tid == 0)
             s_last = (__hip_atomic_fetch_add(counters + tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KS - 1);
@@ -843,23 +849,23 @@ extern "C" int kiln_w4a16_debug_timeline(long long *buf) {
 
 size_t prefill_aext_bytes(int m, int k) { return (size_t)m * (k / kGroupK) * sizeof(u32x4); }
 
-// Scratch of the projection.  For the small-M kernels (up to 128 rows): 16 K slices of T in bf16.
+// Scratch of the projection.  For the small-M kernels (few_rows): up to 16 K slices of T in bf16.
 // For the matrix-core kernel: T once and behind it the f32 tiles in which the slices meet (at most
 // ceil(256 / row tiles) slices per row tile: fewer than 256 + 2 x row tiles tiles of 64 or 16 rows
-// x 64 columns).  Either kernel may get any row count, so the larger of the two.
+// x 64 columns).
 constexpr int kProjectMaxCounters = 16384;
 // measured at 2048 rows: 16-row blocks 9.9 us against 13.1 for K = 2560, 23.5 against 20.2 for K = 9216
 int lora_project_rows_per_block(int m, int k) { return m > 1024 && k > 4096 ? 64 : 16; }
-int prefill_lora_max_slices(int m) { return m <= 128 ? 16 : 1; }
-size_t prefill_lora_t_bytes(int m) {
-    const size_t few = (size_t)prefill_lora_max_slices(m) * m * 64 * sizeof(uint16_t);
+int prefill_lora_max_slices(int) { return 16; }
+size_t prefill_lora_t_bytes(int m, bool few_rows) {
+    if (few_rows) return (size_t)prefill_lora_max_slices(m) * m * 64 * sizeof(uint16_t);
     size_t many = 0;
     for (int rb = 16; rb <= 64; rb *= 4) {  // either block height
         const size_t tiles = 256 + 2 * (size_t)((m + rb - 1) / rb);
         const size_t bytes = (size_t)m * 64 * sizeof(uint16_t) + tiles * rb * 64 * sizeof(float);
         if (bytes > many) many = bytes;
     }
-    return few > many ? few : many;
+    return many;
 }
 
 // Rows of the die grid: the largest power of two up to 8 that divides the row blocks, so that

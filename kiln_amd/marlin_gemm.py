@@ -26,8 +26,9 @@ def _bail(msg: str):
     raise MarlinGemmError(f"kiln-marlin-gemm: {msg}")
 
 
-# one zero-initialised workspace per (device, stream): the kernels leave the
-# counter region zero on exit, so it is allocated once and reused
+# One workspace per (device, stream): only its counter prefix must be zero on first use and the
+# kernels leave it zero on exit, so it is allocated once, grown when a larger call comes, and
+# never cleared again.
 _workspaces: dict[tuple[int, int], torch.Tensor] = {}
 
 
@@ -35,7 +36,8 @@ def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> torch.Tens
     key = (device.index if device.index is not None else torch.cuda.current_device(), stream_ptr)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
-        ws = torch.zeros(nbytes, dtype=torch.uint8, device=device)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=device)
+        ws[:_lib.load().kiln_w4a16_workspace_zeroed_bytes()].zero_()
         _workspaces[key] = ws
     return ws
 
@@ -95,7 +97,11 @@ def marlin_w4a16_gemm(a: torch.Tensor, b_packed: torch.Tensor, scales: torch.Ten
         return out
     with torch.cuda.device(a.device):
         stream = torch.cuda.current_stream(a.device).cuda_stream
-        ws = _workspace(a.device, stream, lib.kiln_w4a16_workspace_bytes(m, n, k))
+        if thread_k > 0 or thread_n > 0:
+            nbytes = lib.kiln_w4a16_workspace_bytes_tuned(m, n, k, thread_k, thread_n, -1)
+        else:
+            nbytes = lib.kiln_w4a16_workspace_bytes(m, n, k)
+        ws = _workspace(a.device, stream, nbytes)
         status = lib.kiln_marlin_w4a16_gemm(
             a.data_ptr(), b_packed.data_ptr(), out.data_ptr(), scales.data_ptr(), m, n, k,
             ws.data_ptr(), groupsize, a.device.index or 0, stream, thread_k, thread_n, -1, 16)

@@ -289,7 +289,7 @@ void ko_lora_delta_add_f32(const uint16_t *x_bf16, const uint16_t *a_bf16,
     free(hidden);
 }
 
-/* adapter_merge.rs:639-712 */
+/* forward.rs:110-114, 2789-2819: silu(gate) * up */
 void ko_swiglu_f32(const float *gate, const float *up, size_t count, float *out) {
 #pragma omp parallel for
     for (size_t i = 0; i < count; ++i) {
@@ -298,6 +298,7 @@ void ko_swiglu_f32(const float *gate, const float *up, size_t count, float *out)
     }
 }
 
+/* adapter_merge.rs:639-712 */
 void ko_merge_concat(const float *const *a_list, const float *const *b_list, const int *ranks,
                      const float *weights, int count, int k, int n, float *a_cat,
                      float *b_cat) {

@@ -62,7 +62,7 @@ def test_lora_through_every_small_m_kernel(oracle, mode, m, k, n, ranks):
     """The three small-M kernels (tile-major runs, group-major staged, group-major in registers),
     chosen through the tuning hook."""
     from kiln_amd import _lib
-    lib = _lib.load()
+    lib = _lib.load_tuning()
     lib.kiln_w4a16_debug_decode_group_major(mode)
     try:
         _lora_case(oracle, m, k, n, ranks, tuple(0.5 + i for i in range(len(ranks))), seed=m + k, sigma_ab=0.05)

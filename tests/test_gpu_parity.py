@@ -149,7 +149,7 @@ def test_forced_decode_plans_agree(oracle, m, k, n, waves, run, kslices):
     (runs of up to 12 chunks, tiles cut by block boundaries, up to 8 slices), with and without
     the LDS staging of the activations: all must match the oracle."""
     from kiln_amd import _lib
-    L = _lib.load()
+    L = _lib.load_tuning()
     x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=waves * 100 + run)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
     try:
@@ -184,7 +184,7 @@ def test_every_tile_major_instance(oracle, run, gs):
     boundary, activations staged in LDS and read directly: each instance is separate
     straight-line code with its own hand-counted waits."""
     from kiln_amd import _lib
-    L = _lib.load()
+    L = _lib.load_tuning()
     m, k, n = 3, gs * 128, 512
     x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=run * 40 + gs)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
@@ -220,7 +220,7 @@ def test_every_group_major_instance(oracle, waves, gpw, tiles):
     register-fragment instance with one and with two slabs of rows.  Each instance is separate
     straight-line code with its own hand-counted waits, so each one is checked."""
     from kiln_amd import _lib
-    L = _lib.load()
+    L = _lib.load_tuning()
     k, n = waves * gpw * 128, 256
     x5, q, s_bits = oracle.gen_problem(5, k, n, 128, seed=waves * 100 + gpw * 10 + tiles)
     x20 = oracle.gen_problem(20, k, n, 128, seed=waves + gpw + tiles)[0]
@@ -424,7 +424,7 @@ def test_rows_33_to_64_through_either_kernel(oracle, m, k, n):
     the last slab ragged); pinned to the matrix-core kernel the same problem must meet the
     same bound."""
     from kiln_amd import _lib
-    L = _lib.load()
+    L = _lib.load_tuning()
     x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=m * 7 + n)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
     _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
@@ -443,7 +443,7 @@ def test_several_runs_of_rows_in_one_launch(oracle, m, k, n):
     per run).  The result must meet
     the oracle bound and, where one launch per run would take the same instance, equal it bit for bit."""
     from kiln_amd import _lib
-    L = _lib.load()
+    L = _lib.load_tuning()
     x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=m * 3 + n)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
     bt, st = upload_packed(b, s)
@@ -476,7 +476,7 @@ def test_every_prefill_block_shape(oracle, bm, bn):
     some of them): each is pinned through the library's tuning hook and must meet the oracle
     bound, whole tiles and K-sliced."""
     from kiln_amd import _lib
-    L = _lib.load()
+    L = _lib.load_tuning()
     m, k, n, g = 300, 2560, 2560, 128
     x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=bm + bn, sigma=0.5)
     b, s = pack.repack_gptq(q, s_bits, None, g)

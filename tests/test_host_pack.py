@@ -374,3 +374,57 @@ def test_decode_plans_are_launchable_and_keep_model_shapes_exchange_free():
         ks, gs, u, bps, waves, _, regs, gm_tiles = list(out)
         assert ks * gs == 72 and (gm_tiles or (waves * u) % gs == 0) and ks * bps <= 256 and regs == (m > 16), list(out)
     assert plan(33, 2560, 2560, 256, out) == 1 and plan(16, 2560, 100, 256, out) == 1
+
+
+MODEL_SHAPES = [(2560, 8192), (4096, 2560), (2560, 18432), (9216, 2560)]      # (k, n)
+
+
+@pytest.mark.parametrize("k,n", MODEL_SHAPES)
+def test_workspace_bytes_is_monotone_in_m(k, n):
+    """A workspace sized for the largest m must serve every smaller call: the size function is
+    the running maximum of the per-call need, so it never decreases with m (m = 1...8192 on the
+    model's four projection shapes), and it starts at no less than the zeroed counter prefix."""
+    L = _lib.load()
+    sizes = [L.kiln_w4a16_workspace_bytes(m, n, k) for m in range(1, 8193)]
+    assert sizes[0] >= L.kiln_w4a16_workspace_zeroed_bytes()
+    drops = [(m + 1, sizes[m - 1], sizes[m]) for m in range(1, len(sizes)) if sizes[m] < sizes[m - 1]]
+    assert not drops, drops[:5]
+    # with overrides the sizing takes them into account and is monotone as well
+    tuned = [L.kiln_w4a16_workspace_bytes_tuned(m, n, k, 128, 16, -1) for m in range(1, 200)]
+    assert all(b >= a for a, b in zip(tuned, tuned[1:]))
+    assert tuned[15] >= sizes[15] or tuned[15] >= L.kiln_w4a16_workspace_zeroed_bytes()
+
+
+def test_workspace_is_small_where_nothing_is_exchanged():
+    """Decode calls on the projections whose plan exchanges nothing through the workspace need
+    little more than the counters and the LoRA projection scratch; the down projection's three
+    K slices need their partial tiles and no more."""
+    L = _lib.load()
+    z = L.kiln_w4a16_workspace_zeroed_bytes()
+    assert z == 64 * 1024
+    for k, n in [(2560, 8192), (4096, 2560), (2560, 18432)]:
+        assert L.kiln_w4a16_workspace_bytes(16, n, k) <= z + 64 * 1024, (k, n)
+    down = L.kiln_w4a16_workspace_bytes(16, 2560, 9216)
+    assert z + 3 * 2 * 2560 * 64 <= down <= z + 3 * 2 * 2560 * 64 + 64 * 1024
+
+
+def test_shipped_library_has_no_tuning_setters():
+    """The plan overrides exist only in the tuning build; the shipped library exports none."""
+    shipped, tuning = _lib.load(), _lib.load_tuning()
+    for name in _lib.TUNING_EXPORTS:
+        assert not hasattr(shipped, name), name
+        assert hasattr(tuning, name), name
+    for name in _lib.EXPORTS + _lib.PROJ_EXPORTS:
+        assert hasattr(shipped, name) and hasattr(tuning, name), name
+
+
+def test_long_k_falls_back_to_the_matrix_core_path():
+    """K beyond eight slices of 32 groups has no small-M plan; such a GEMM takes the matrix-core
+    kernel at any row count instead of failing (the reference accepts any k % 128 == 0)."""
+    L = _lib.load()
+    out = (ctypes.c_int * 8)()
+    for k in (32896, 40960):
+        for m in (1, 16, 48):
+            assert L.kiln_w4a16_debug_gemm_plan(m, 2560, k, 256, out) == 0
+            assert out[0] == 1, (m, k, list(out))
+    assert L.kiln_w4a16_debug_gemm_plan(16, 2560, 9216, 256, out) == 0 and out[0] == 0 and out[1] == 1
