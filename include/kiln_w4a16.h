@@ -46,6 +46,10 @@ typedef int kiln_marlin_status_t;
 #define KILN_W4A16_ERR_LAUNCH       3  /* HIP reported an error at launch */
 #define KILN_W4A16_ERR_ARGUMENT     4  /* null pointer or inconsistent argument */
 #define KILN_W4A16_ERR_ZERO_POINT   5  /* repack: a GPTQ zero-point other than 8 */
+#define KILN_W4A16_ERR_SCRATCH      6  /* the call needs more scratch than the library's static array holds */
+
+/* Size of the static device array behind kiln_marlin_w4a16_gemm_static_scratch (per GPU). */
+#define KILN_W4A16_STATIC_SCRATCH_BYTES (4u << 20)
 
 /*
  * C = A * dequant(B, s).
@@ -90,6 +94,25 @@ size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k,
  * reference's whole lock array has that contract, marlin_kernel.cu:177-180, lib.rs:176-178).
  */
 size_t kiln_w4a16_workspace_zeroed_bytes(void);
+
+/*
+ * kiln_marlin_w4a16_gemm without the workspace argument, for callers that cannot allocate
+ * device memory or hand a workspace over: code running under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its wrapper
+ * allocates and zero-fills a workspace per call, lib.rs:174-178).  The counters and f32 partial
+ * tiles live in a device array inside the library, KILN_W4A16_STATIC_SCRATCH_BYTES = 4 MiB per
+ * GPU the library runs on, held until the process ends.  The call allocates nothing and frees
+ * nothing.  A shape whose plan needs more than that (kiln_w4a16_workspace_bytes says how much a
+ * shape needs; every decode call of the model's projections, m <= 80, needs at most 2.3 MB; large
+ * K-sliced prefill calls need tens of MB) is refused with KILN_W4A16_ERR_SCRATCH before anything
+ * is launched.  `dev` must be the current device.  All calls on one GPU share that GPU's array:
+ * calls that may overlap in time (different streams, or threads launching concurrently) race on
+ * it and must be ordered by the caller; calls on one stream are safe back to back.
+ */
+kiln_marlin_status_t kiln_marlin_w4a16_gemm_static_scratch(
+    const void *A, const void *B, void *C, void *s,
+    int prob_m, int prob_n, int prob_k,
+    int groupsize, int dev, void *stream);
 
 /*
  * C = A * dequant(B, s) + sum_i scale_i * (A * lora_a_i^T) * lora_b_i^T.  Fuses what

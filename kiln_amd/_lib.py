@@ -16,6 +16,7 @@ EXPORTS = (
     "kiln_w4a16_workspace_bytes",
     "kiln_w4a16_workspace_bytes_tuned",
     "kiln_w4a16_workspace_zeroed_bytes",
+    "kiln_marlin_w4a16_gemm_static_scratch",
     "kiln_w4a16_gemm_lora",
     "kiln_w4a16_gemm_swiglu",
     "kiln_w4a16_swiglu_workspace_bytes",
@@ -53,7 +54,9 @@ PROJ_EXPORTS = (
 
 PROJ_OK, PROJ_SKIPPED, PROJ_ERR = 0, 1, -1
 
-OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_LAUNCH, ERR_ARGUMENT, ERR_ZERO_POINT = range(6)
+STATIC_SCRATCH_BYTES = 4 << 20   # KILN_W4A16_STATIC_SCRATCH_BYTES
+
+OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_LAUNCH, ERR_ARGUMENT, ERR_ZERO_POINT, ERR_SCRATCH = range(7)
 
 # The tuning build: the same sources with -DKILN_W4A16_TUNING_HOOKS, which adds process-wide
 # overrides of the automatic plan (kiln_w4a16_debug_*).  Tests and profiling scripts that pin a
@@ -129,6 +132,8 @@ def _load(tuning: bool) -> ctypes.CDLL:
     L.kiln_w4a16_workspace_bytes_tuned.argtypes = [i, i, i, i, i, i]
     L.kiln_w4a16_workspace_zeroed_bytes.restype = c.c_size_t
     L.kiln_w4a16_workspace_zeroed_bytes.argtypes = []
+    L.kiln_marlin_w4a16_gemm_static_scratch.restype = i
+    L.kiln_marlin_w4a16_gemm_static_scratch.argtypes = [vp, vp, vp, vp, i, i, i, i, i, vp]
     L.kiln_w4a16_debug_decode_plan.restype = i
     L.kiln_w4a16_debug_decode_plan.argtypes = [i, i, i, i, c.POINTER(c.c_int)]
     L.kiln_w4a16_debug_gemm_plan.restype = i

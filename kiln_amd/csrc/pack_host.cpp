@@ -111,6 +111,9 @@ const char *kiln_w4a16_status_string(kiln_marlin_status_t st) {
         case KILN_W4A16_ERR_LAUNCH: return "HIP launch error";
         case KILN_W4A16_ERR_ARGUMENT: return "null or inconsistent argument";
         case KILN_W4A16_ERR_ZERO_POINT: return "GPTQ zero-point other than 8 is not supported";
+        case KILN_W4A16_ERR_SCRATCH:
+            return "the call needs more scratch than the library's static device array holds; use the entry point "
+                   "that takes a workspace";
         default: return "unknown status";
     }
 }

@@ -375,10 +375,11 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, GemmPla
     }
 }
 
-// workspace of one call: counters | small-M partial tiles | LoRA projection           (small-M path)
-//                        counters | row-sum operands | LoRA projection | partial tiles (matrix-core path)
+// workspace of one call: counters | small-M partial tiles | LoRA projection             (small-M path)
+//                        counters | row-sum operands | partial tiles | LoRA projection (matrix-core path)
+// The LoRA projection's scratch comes last: a call without adapters needs `plain` bytes only.
 struct WorkspaceLayout {
-    size_t decode_partial, aext, lora_t, prefill_partial, total;
+    size_t decode_partial, aext, lora_t, prefill_partial, plain, total;
 };
 WorkspaceLayout workspace_layout(const GemmPlan &gp, int m, int n, int k) {
     WorkspaceLayout w{};
@@ -386,18 +387,17 @@ WorkspaceLayout workspace_layout(const GemmPlan &gp, int m, int n, int k) {
     if (gp.prefill) {
         w.aext = off;
         off += prefill_aext_bytes(m, k);
-        w.lora_t = off;
-        off += prefill_lora_t_bytes(m, false);
         off = (off + 255) & ~(size_t)255;
         w.prefill_partial = off;
         off += prefill_partial_bytes(m, n, gp.pf);
     } else {
         w.decode_partial = off;
         off += gp.decode_partial;
-        off = (off + 255) & ~(size_t)255;
-        w.lora_t = off;
-        off += prefill_lora_t_bytes(m, true);
     }
+    w.plain = off;
+    off = (off + 255) & ~(size_t)255;
+    w.lora_t = off;
+    off += prefill_lora_t_bytes(m, !gp.prefill);
     w.total = off;
     return w;
 }
@@ -605,6 +605,63 @@ size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k, int 
 }
 
 size_t kiln_w4a16_workspace_zeroed_bytes(void) { return kCounterBytes; }
+
+// ---- the GEMM for callers that cannot hand over (or allocate) a workspace ----------------------
+// The workspace of kiln_marlin_w4a16_gemm -- arrival counters and the f32 partial tiles of K-sliced
+// launches -- lives in a device array of the library instead.  Each GPU the library runs on holds
+// its own copy at its own address until the process ends; the loader zero-fills it, and every call
+// leaves the counter prefix zero again.  In host code the array's name is only a handle: the
+// address kernels may use comes from hipGetSymbolAddress, asked once per device with that device
+// current, and is what every launch gets as its workspace argument.
+}  // extern "C"
+
+namespace kiln {
+namespace {
+
+constexpr size_t kStaticScratchBytes = KILN_W4A16_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+struct StaticScratch {
+    std::once_flag once;
+    void *ptr = nullptr;
+    hipError_t err = hipErrorNotInitialized;
+};
+StaticScratch g_static_scratch[kMaxDevices];
+
+// device address of the current device's copy of `scratch` (nullptr if the runtime refuses)
+void *static_scratch_ptr(int current_dev) {
+    StaticScratch &slot = g_static_scratch[current_dev];
+    std::call_once(slot.once, [&]() {
+        void *p = nullptr;
+        slot.err = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (slot.err == hipSuccess) slot.ptr = p;
+    });
+    return slot.err == hipSuccess ? slot.ptr : nullptr;
+}
+
+}  // namespace
+}  // namespace kiln
+
+extern "C" {
+
+kiln_marlin_status_t kiln_marlin_w4a16_gemm_static_scratch(const void *A, const void *B, void *C, void *s,
+                                                           int prob_m, int prob_n, int prob_k, int groupsize,
+                                                           int dev, void *stream) {
+    if (prob_m < 0 || prob_n < 0 || prob_k < 0) return KILN_W4A16_ERR_PROB_SHAPE;
+    if (!shape_ok(prob_n, prob_k, groupsize)) return KILN_W4A16_ERR_PROB_SHAPE;
+    if (prob_m == 0 || prob_n == 0 || prob_k == 0) return KILN_W4A16_OK;
+    if (!A || !B || !C || !s) return KILN_W4A16_ERR_ARGUMENT;
+    // the array belongs to the device that is current: that must be the one the caller names
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current != dev || dev < 0 || dev >= kMaxDevices)
+        return KILN_W4A16_ERR_ARGUMENT;
+    GemmPlan gp;
+    plan_gemm(prob_m, prob_n, prob_k, compute_units(dev), -1, -1, &gp);
+    if (workspace_layout(gp, prob_m, prob_n, prob_k).plain > kStaticScratchBytes) return KILN_W4A16_ERR_SCRATCH;
+    void *ws = static_scratch_ptr(current);
+    if (!ws) return KILN_W4A16_ERR_LAUNCH;
+    return gemm_any(A, B, C, s, prob_m, prob_n, prob_k, ws, groupsize, dev, stream, -1, -1, -1, nullptr);
+}
 
 kiln_marlin_status_t kiln_marlin_w4a16_gemm(const void *A, const void *B, void *C, void *s,
                                             int prob_m, int prob_n, int prob_k, void *workspace,

@@ -195,3 +195,26 @@ def test_lora_argument_errors():
         marlin_gemm.marlin_w4a16_gemm_lora(a, b, s, 128, big_a, big_b, [72], [1.0])   # rank > 64
     y = marlin_gemm.marlin_w4a16_gemm_lora(a, b, s, 128, la, lb, [8], [1.0])
     assert tuple(y.shape) == (2, 256)
+
+
+@pytest.mark.parametrize("m,k,n,ranks", [(200, 9216, 256, (7,)), (16, 9216, 2560, (16, 32))])
+def test_lora_run_to_run_determinism(oracle, m, k, n, ranks):
+    """The projection's K slices meet as f32 tiles in the workspace (many rows) and the GEMM's own
+    K slices exchange partial tiles (few rows): 1000 launches, identical bits, stopping at the
+    first difference."""
+    g = 128
+    x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=m)
+    b, s = pack.repack_gptq(q, s_bits, None, g)
+    bt, st = upload_packed(b, s)
+    a_cat = bf16_tensor(np.concatenate([oracle.gen_normal_bf16(r, k, 0.05, seed=40 + i) for i, r in enumerate(ranks)], axis=0))
+    b_cat = bf16_tensor(np.concatenate([oracle.gen_normal_bf16(n, r, 0.05, seed=50 + i) for i, r in enumerate(ranks)], axis=1))
+    scales = tuple(1.0 for _ in ranks)
+    xt = bf16_tensor(x)
+    first = marlin_gemm.marlin_w4a16_gemm_lora(xt, bt, st, g, a_cat, b_cat, ranks, scales).clone()
+    out = torch.empty_like(first)
+    same = torch.ones((), dtype=torch.bool, device=first.device)
+    for i in range(1000):
+        marlin_gemm.marlin_w4a16_gemm_lora(xt, bt, st, g, a_cat, b_cat, ranks, scales, out=out)
+        same &= (out == first).all()
+        if i % 50 == 49:
+            assert bool(same), f"launch {i - 49}...{i} differed from the first"
