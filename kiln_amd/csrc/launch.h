@@ -64,6 +64,25 @@ bool decode_group_major_regs_ok(const struct DecodeArgs &a);  // ... and the one
 int decode_max_tiles_per_block();
 hipError_t launch_decode(const DecodeArgs &args, hipStream_t stream);
 
+// One launch of the mid-M kernel: runs of up to 64 rows (grid z) against the whole weight.
+struct MidArgs {
+    const void *A;      // bf16 [M, K]
+    const void *B;      // packed weights, tile layout
+    const void *S;      // fp16 scales, tile layout
+    void *C;            // bf16 [M, N]
+    float *partial;     // mid_partial_bytes() bytes when KS > 1
+    int *counters;      // runs * N / (32 * pairs) arrival counters, zero on entry and on exit
+    int M, N, K, Gs;
+    int KS;             // K slices, all of GS groups
+    int GS;             // 128-row groups per slice
+    int waves;          // wavefronts per block, <= 8 and <= GS; each owns ceil(GS / waves) groups or one fewer
+    int pairs;          // pairs of 16-column tiles per block: 1 or 2
+};
+int mid_max_rows_per_run();
+bool mid_plan_ok(const MidArgs &a);
+size_t mid_partial_bytes(const MidArgs &a);
+hipError_t launch_mid(const MidArgs &a, hipStream_t stream);
+
 // One launch of the prefill path (row-sum pre-pass + MFMA kernel), any M >= 1.
 struct PrefillArgs {
     const void *A;   // bf16 [M, K]

@@ -61,6 +61,8 @@ struct Tuning {
     int decode_runs_per_launch = 0;   // 1 = one run of rows per launch
     int prefill_ks = 0, prefill_bn = 0, prefill_bm = 0, prefill_nb_full = -1;
     int force_ks = 0, force_u = 0, force_waves = 0;
+    int mid = -1;                     // 0 = never the mid-M kernel, 1 = wherever a plan fits (any row count), -1 = automatic
+    int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
 };
 #ifdef KILN_W4A16_TUNING_HOOKS
 Tuning g_tune;
@@ -291,9 +293,16 @@ struct DecodeLaunch {
     DecodePlan plan;
     bool direct;
 };
+struct MidPlan {
+    bool ok = false;
+    int KS = 1, GS = 0, waves = 0, pairs = 1;
+    float cost = 0.f;
+};
 struct GemmPlan {
     bool prefill = false;
     PrefillPlan pf{};
+    bool mid = false;
+    MidPlan mp{};
     int launches = 0;
     DecodeLaunch dl[kMaxDecodeLaunches];
     size_t decode_partial = 0;  // bytes of partial tiles the largest launch exchanges
@@ -332,8 +341,73 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
     gp->pf = p;
 }
 
-void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, GemmPlan *gp) {
+// Rows the mid-M kernel takes on the automatic plan: above the two-slab small-M instance's 32 and
+// up to two runs of 64.
+constexpr int kMidMinM = 33, kMidMaxM = 128;
+
+// Plan for the mid-M kernel: pairs of tiles per block, K slices, wavefronts.  Cost in microseconds,
+// from the kernel's arithmetic: a wavefront issues 16 products per pair and 16 for the offset tile
+// per group, 32 cycles each at about 2.3 GHz, two wavefronts per SIMD above four per block; a
+// round of blocks costs about 1 us beside its products (first loads, reduction), an exchange
+// between K slices 2.2 us plus 0.1 us per slice.
+MidPlan plan_mid(int m, int n, int k, int cus) {
+    MidPlan best;
+    const int G = k / kGroupK, NT = n / kTileN, runs = ceil_div(m, mid_max_rows_per_run());
+    for (int pairs = 1; pairs <= 2; ++pairs) {
+        if (g_tune.mid_pairs && pairs != g_tune.mid_pairs) continue;
+        for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
+            if (G % ks != 0 || (g_tune.mid_ks && ks != g_tune.mid_ks)) continue;
+            MidArgs a{};
+            a.M = m;
+            a.N = n;
+            a.K = k;
+            a.KS = ks;
+            a.GS = G / ks;
+            a.waves = a.GS < 8 ? a.GS : 8;
+            a.pairs = pairs;
+            if (!mid_plan_ok(a)) continue;
+            const int col_blocks = NT / (2 * pairs);
+            if ((size_t)runs * col_blocks * sizeof(int) > kCounterBytes) continue;
+            const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
+            const float t_block = (float)ceil_div(a.waves, 4) * gpw * (pairs + 1) * 0.2226f;
+            const float cost = rounds * (t_block + 1.0f) + (ks > 1 ? 2.2f + 0.1f * ks : 0.f);
+            if (!best.ok || cost < best.cost) {
+                best.ok = true;
+                best.KS = ks;
+                best.GS = a.GS;
+                best.waves = a.waves;
+                best.pairs = pairs;
+                best.cost = cost;
+            }
+        }
+    }
+    return best;
+}
+
+MidArgs mid_args(const MidPlan &mp, int m, int n, int k) {
+    MidArgs a{};
+    a.M = m;
+    a.N = n;
+    a.K = k;
+    a.KS = mp.KS;
+    a.GS = mp.GS;
+    a.waves = mp.waves;
+    a.pairs = mp.pairs;
+    return a;
+}
+
+void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, bool lora, GemmPlan *gp) {
     *gp = GemmPlan{};
+    // 33...128 rows of a plain GEMM: the mid-M kernel, one pass over the weights per 64 rows
+    if (!lora && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
+        (g_tune.mid == 1 || (g_tune.prefill_min_m == 0 && m >= kMidMinM && m <= kMidMaxM))) {
+        const MidPlan mp = plan_mid(m, n, k, cus);
+        if (mp.ok) {
+            gp->mid = true;
+            gp->mp = mp;
+            return;
+        }
+    }
     // the small-M kernels keep one arrival counter per column tile (and run) in the counter region
     const bool counters_fit = (size_t)(n / kTileN) * sizeof(int) <= kCounterBytes;
     if (!counters_fit || takes_prefill(m, n, k, cus)) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
@@ -392,7 +466,7 @@ WorkspaceLayout workspace_layout(const GemmPlan &gp, int m, int n, int k) {
         off += prefill_partial_bytes(m, n, gp.pf);
     } else {
         w.decode_partial = off;
-        off += gp.decode_partial;
+        off += gp.mid ? mid_partial_bytes(mid_args(gp.mp, m, n, k)) : gp.decode_partial;
     }
     w.plain = off;
     off = (off + 255) & ~(size_t)255;
@@ -475,10 +549,12 @@ struct LoraSpec {
 size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thread_n) {
     size_t most = 0;
     auto consider = [&](int mm) {
-        GemmPlan gp;
-        plan_gemm(mm, n, k, cus, thread_k, thread_n, &gp);
-        const size_t need = workspace_layout(gp, mm, n, k).total;
-        if (need > most) most = need;
+        for (int lora = 0; lora < 2; ++lora) {  // a call with adapters may take another path
+            GemmPlan gp;
+            plan_gemm(mm, n, k, cus, thread_k, thread_n, lora != 0, &gp);
+            const size_t need = workspace_layout(gp, mm, n, k).total;
+            if (need > most) most = need;
+        }
     };
     const int small = g_tune.prefill_min_m > 128 ? g_tune.prefill_min_m : 128;
     for (int mm = 1; mm <= m && mm <= small; ++mm) consider(mm);
@@ -502,7 +578,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     const int cus = sms > 0 ? sms : compute_units(dev);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     GemmPlan gp;
-    plan_gemm(prob_m, prob_n, prob_k, cus, thread_k, thread_n, &gp);
+    plan_gemm(prob_m, prob_n, prob_k, cus, thread_k, thread_n, lora != nullptr, &gp);
     const WorkspaceLayout wl = workspace_layout(gp, prob_m, prob_n, prob_k);
     char *ws = reinterpret_cast<char *>(workspace);
     char *lora_t = ws + wl.lora_t;
@@ -534,6 +610,18 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         pa.counters = reinterpret_cast<int *>(workspace);
         pa.partial = reinterpret_cast<float *>(ws + wl.prefill_partial);
         return launch_prefill(pa, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+    }
+
+    if (gp.mid) {
+        MidArgs ma = mid_args(gp.mp, prob_m, prob_n, prob_k);
+        ma.A = A;
+        ma.B = B;
+        ma.S = s;
+        ma.C = C;
+        ma.Gs = (groupsize == -1) ? 1 : prob_k / kGroupK;
+        ma.counters = reinterpret_cast<int *>(workspace);
+        ma.partial = reinterpret_cast<float *>(ws + wl.decode_partial);
+        return launch_mid(ma, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
     }
 
     int rp = 0, lora_slices = 1;
@@ -656,7 +744,7 @@ kiln_marlin_status_t kiln_marlin_w4a16_gemm_static_scratch(const void *A, const 
     if (hipGetDevice(&current) != hipSuccess || current != dev || dev < 0 || dev >= kMaxDevices)
         return KILN_W4A16_ERR_ARGUMENT;
     GemmPlan gp;
-    plan_gemm(prob_m, prob_n, prob_k, compute_units(dev), -1, -1, &gp);
+    plan_gemm(prob_m, prob_n, prob_k, compute_units(dev), -1, -1, false, &gp);
     if (workspace_layout(gp, prob_m, prob_n, prob_k).plain > kStaticScratchBytes) return KILN_W4A16_ERR_SCRATCH;
     void *ws = static_scratch_ptr(current);
     if (!ws) return KILN_W4A16_ERR_LAUNCH;
@@ -688,13 +776,16 @@ int kiln_w4a16_debug_decode_plan(int m, int n, int k, int cus, int *out) {
 }
 
 // Which path a plain GEMM takes (a pure query, not part of the public header):
-// out = {matrix-core path?, launches, block rows, block columns, whole column blocks, K slices}.
+// out = {matrix-core path?, small-M launches, block rows, block columns, whole column blocks, K slices,
+//        mid-M kernel?, its tile pairs * 16 + K slices}.
 int kiln_w4a16_debug_gemm_plan(int m, int n, int k, int cus, int *out) {
     if (m < 1 || cus < 1 || !shape_ok(n, k, 128)) return 1;
     GemmPlan gp;
-    plan_gemm(m, n, k, cus, -1, -1, &gp);
+    plan_gemm(m, n, k, cus, -1, -1, false, &gp);
     out[0] = gp.prefill; out[1] = gp.launches; out[2] = gp.pf.bm; out[3] = gp.pf.bn; out[4] = gp.pf.nb_full;
     out[5] = gp.pf.ks;
+    out[6] = gp.mid;          // the mid-M kernel: pairs of tiles per block, K slices
+    out[7] = gp.mid ? gp.mp.pairs * 16 + gp.mp.KS : 0;
     return 0;
 }
 
@@ -714,6 +805,11 @@ void kiln_w4a16_debug_prefill_nb_full(int nb) { g_tune.prefill_nb_full = nb; }
 void kiln_w4a16_debug_decode_direct_max_m(int m) { g_tune.decode_direct_max_m = m; tuning_changed(); }
 void kiln_w4a16_debug_decode_group_major(int mode) { g_tune.decode_group_major = mode; tuning_changed(); }
 void kiln_w4a16_debug_decode_runs_per_launch(int runs) { g_tune.decode_runs_per_launch = runs; }
+void kiln_w4a16_debug_mid(int mode, int pairs, int kslices) {
+    g_tune.mid = mode;
+    g_tune.mid_pairs = pairs;
+    g_tune.mid_ks = kslices;
+}
 void kiln_w4a16_debug_tune(int waves, int run, int kslices) {
     g_tune.force_waves = waves;
     g_tune.force_u = run;

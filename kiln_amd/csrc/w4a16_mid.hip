@@ -1,0 +1,371 @@
+// Mid-M W4A16 GEMM kernel for gfx950: runs of up to 64 rows per pass over the weights.
+//
+// Covers the row counts between the decode kernels (one or two 16-row slabs, 16x16x32
+// products) and the prefill kernel (whole-chip tiling, matrix-core bound): the arm of the
+// reference dispatcher that pads M to 16 * thread_m_blocks up to 64 rows
+// (crates/kiln-marlin-gemm/csrc/marlin_kernel.cu:784-816).  At 33...128 rows the problem is
+// still bound by the int4 weight stream, but the products are no longer free: 64 rows take
+// v_mfma_f32_32x32x16_bf16 (the 16-row shape runs at half the rate per flop) and one pass over
+// the weights.
+//
+// Work split (group-major, as in the decode kernels): a block owns TP pairs of neighbouring
+// 16-column tiles (32 columns per pair = one 32x32 product tile) and one K slice of GS groups;
+// wavefront w owns a contiguous run of those groups and multiplies them with every pair of the
+// block, 64 rows each.  So each element of the activations is read once per block, by the one
+// wavefront that needs it, and nobody waits at a barrier before the first product:
+//   * A: the wavefront's 64 rows x 128 values of one group go from L2 into its private 16 KiB
+//     of LDS with 16 LDS-direct loads (4 rows of 256 bytes each, fully coalesced), swizzled on
+//     16-byte units so that the fragment reads are free of bank conflicts; the fragments are
+//     then held in registers for the whole group, which frees the LDS slot for the next group.
+//   * B: 2 x 128-bit per lane, pair and group, straight into the product's operand layout,
+//     requested one or two groups ahead (as the registers allow) into rotating register sets.
+//   * Scales in f32 by a running rescale of the accumulators (as in the prefill kernel); the
+//     B operand carries 136 + d, and the surplus is removed by an offset tile per group and row
+//     block (eight products with a constant -136 operand, shared by all pairs) that enters the
+//     rescale as the addend of one fused multiply-add per accumulator register.
+// At the end the wavefronts' f32 tiles are summed through LDS in wavefront (= ascending K)
+// order; K slices of a tile meet in the workspace, last arriver adds in slice order.
+#include "async_loads.h"
+#include "launch.h"
+
+namespace kiln {
+
+namespace {
+
+constexpr int kMidWaves = 8;                    // wavefronts per block, at most
+constexpr int kMidRows = 64;                    // rows per run
+constexpr int kMidSlotBytes = kMidRows * 256;   // one group of A: 64 rows x 128 bf16
+constexpr int kMidALoads = 16;                  // LDS-direct loads per group of A
+constexpr int kMidMaxGroups = 4;                // groups per wavefront, at most
+
+// Issue order of a wavefront's loads -- A(g): 16 LDS-direct loads, B(g): NL register loads, the
+// weights D groups ahead in D + 1 register sets --
+//   before the first step: A(0), B(0) ... B(D-1);
+//   step g: [wait for A(g)] fragments to registers, A(g+1), B(g+D), [wait for B(g)], products.
+// wait_a[g] / wait_b[g] = loads issued after A(g) / B(g) up to that wait: what may still be
+// outstanding when the wait returns.
+struct MidSchedule {
+    int wait_a[kMidMaxGroups];
+    int wait_b[kMidMaxGroups];
+};
+constexpr MidSchedule mid_schedule(int ng, int nl, int d) {
+    int kind[4 * kMidMaxGroups] = {}, grp[4 * kMidMaxGroups] = {}, size[4 * kMidMaxGroups] = {};
+    int n = 0;
+    auto push = [&](int k, int g, int sz) {
+        kind[n] = k;
+        grp[n] = g;
+        size[n] = sz;
+        ++n;
+    };
+    auto issued_after = [&](int k, int g) {
+        int after = 0;
+        bool seen = false;
+        for (int i = 0; i < n; ++i) {
+            if (seen) after += size[i];
+            if (kind[i] == k && grp[i] == g) seen = true;
+        }
+        return after;
+    };
+    push(0, 0, kMidALoads);
+    for (int g = 0; g < d && g < ng; ++g) push(1, g, nl);
+    MidSchedule s{};
+    for (int g = 0; g < ng; ++g) {
+        s.wait_a[g] = issued_after(0, g);
+        if (g + 1 < ng) push(0, g + 1, kMidALoads);
+        if (g + d < ng) push(1, g + d, nl);
+        s.wait_b[g] = issued_after(1, g);
+    }
+    return s;
+}
+
+template <int NG, int NL, int D>
+struct MidScheduleOf {
+    static constexpr MidSchedule value = mid_schedule(NG, NL, D);
+};
+
+template <int TP, int GPW>
+__global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
+    const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
+    uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
+    int GS, int full_waves) {
+    extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+    __shared__ int s_last;
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int nw = blockDim.x >> 6;
+    const int l32 = lane & 31, h = lane >> 5;
+    const int G = K / kGroupK;
+    // blockIdx.z: which run of 64 rows (each with its own counters and partial tiles)
+    const int zr = blockIdx.z * kMidRows;
+    const int M = min(rows - zr, kMidRows);
+    const uint16_t *__restrict__ A = A_all + (size_t)zr * K;
+    uint16_t *__restrict__ C = C_all + (size_t)zr * N;
+    const int ks = blockIdx.y;
+    const int tf = blockIdx.x * (2 * TP);  // first 16-column tile of the block
+    // the first `full_waves` wavefronts own GPW groups each, the others GPW - 1
+    const bool full = wave < full_waves;
+    const int g_first = full ? wave * GPW : full_waves * GPW + (wave - full_waves) * (GPW - 1);
+    const int g0 = ks * GS + g_first;  // all slices have GS groups
+    const int gs_mask = (Gs == 1) ? 0 : -1;
+
+    // --- A: 16 loads of 4 rows x 256 bytes.  Lane i of load p fetches 16-byte unit
+    // (i % 16) ^ (row % 16) of row 4 p + i / 16, so unit u of a row sits at position u ^ (row % 16):
+    // the 16 lanes that read one unit index of 16 different rows then hit 16 different positions.
+    // Rows from M on read row M - 1 (a valid address); their products are never stored.
+    unsigned char *slot = lds + wave * kMidSlotBytes;
+    const unsigned slot_addr = (unsigned)(size_t)(lds_ptr_t)slot;
+    const uint32_t row_pitch = (uint32_t)K * 2;
+    auto request_a = [&](int gi) {
+        const char *base = reinterpret_cast<const char *>(A) + (size_t)(g0 + gi) * 256;
+        const uint32_t quad_row = (uint32_t)(lane >> 4) + opaque_zero();  // keeps the offsets below local to this group
+#pragma unroll
+        for (int p = 0; p < kMidALoads; ++p) {
+            const uint32_t row = 4 * p + quad_row;
+            const uint32_t off = min(row, (uint32_t)(M - 1)) * row_pitch + (((uint32_t)(lane & 15) ^ (row & 15)) << 4);
+            load_to_lds_b128(base, off, slot_addr + p * 1024);
+        }
+    };
+
+    // --- B: pair p = tiles tf + 2 p, tf + 2 p + 1.  Lane (l32, h) holds column l32 of the pair and
+    // rows 16 s + 8 h ... + 7 of step s: word s / 2 of the 128-bit unit c + 16 (2 (s % 2) + h) of
+    // chunk l32 / 16 (c = l32 % 16).  Load v = s % 2 therefore serves steps v, v + 2, v + 4, v + 6.
+    constexpr int D = TP == 1 ? 2 : 1;  // groups of look-ahead (two pairs: the registers allow one)
+    constexpr int kSets = D + 1;
+    u32x4 bw[kSets][TP][2];
+    uint32_t sc_raw[kSets][TP];
+    const uint32_t b_lane = (uint32_t)(l32 >> 4) * (uint32_t)G * 1024u + (uint32_t)((l32 & 15) + 16 * h) * 16u;
+    const uint32_t s_lane = (uint32_t)(l32 >> 4) * (uint32_t)Gs * (kTileN * 2) + (uint32_t)(l32 & 15) * 2u;
+    auto request_b = [&](auto gc) {
+        constexpr int gi = decltype(gc)::value, set = gi % kSets;
+        const int g = g0 + gi;
+        unrolled<0, TP>([&](auto pc) {
+            constexpr int p = decltype(pc)::value;
+            const char *bb = reinterpret_cast<const char *>(B) + ((size_t)(tf + 2 * p) * G + g) * 1024;
+            load_b128_streaming(bw[set][p][0], bb, b_lane);
+            load_b128_streaming(bw[set][p][1], bb, b_lane + 512u);
+            const char *sb = reinterpret_cast<const char *>(S) + ((size_t)(tf + 2 * p) * Gs + (g & gs_mask)) * (kTileN * 2);
+            load_u16(sc_raw[set][p], sb, s_lane);
+        });
+    };
+
+    // a zero scale would break the running rescale; it is replaced by a value too small to matter
+    // (the exact result for such a group is 0; the stand-in contributes < 1e-12 * |a|)
+    auto scale_value = [&](uint32_t raw) {
+        const float sv = f16_bits_to_f32((uint16_t)raw);
+        return sv == 0.f ? 0x1p-40f : sv;
+    };
+
+    const bf16x8 minus_bias = bf16x8_splat(0xC308C308u);  // bf16(-136) pairs
+    const DequantConsts dq = dequant_consts();
+    f32x16 acc[TP][2];
+#pragma unroll
+    for (int p = 0; p < TP; ++p)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[p][rb][r] = 0.f;
+
+    // The wavefront's groups: straight-line code from the first request to the last use, one
+    // instance per group count (a register that an asm load fills must be requested, waited for and
+    // used inside one basic block).
+    auto run = [&](auto nc) {
+        constexpr int NG = decltype(nc)::value;
+        constexpr int NL = 3 * TP;
+        using Sch = MidScheduleOf<NG, NL, D>;
+        request_a(0);
+        unrolled<0, (D < NG ? D : NG)>(request_b);
+        float s_cur[TP];
+        unrolled<0, NG>([&](auto gc) {
+            constexpr int gi = decltype(gc)::value, set = gi % kSets;
+            // this group's rows of A are in LDS; their fragments go to registers: lane (l32, h) holds
+            // row 32 rb + l32, values 16 s + 8 h ... + 7 of the group
+            wait_vector_loads<Sch::value.wait_a[gi]>();
+            u32x4 af[2][8];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int s = 0; s < 8; ++s)
+                    af[rb][s] = *reinterpret_cast<const u32x4 *>(slot + (rb * 32 + l32) * 256 +
+                                                                 (((2 * s + h) ^ (l32 & 15)) << 4));
+            wait_lds_reads();  // the slot is free again
+            if constexpr (gi + 1 < NG) request_a(gi + 1);
+            if constexpr (gi + D < NG) request_b(std::integral_constant<int, gi + D>{});
+            wait_vector_loads<Sch::value.wait_b[gi]>();
+            float f[TP];
+#pragma unroll
+            for (int p = 0; p < TP; ++p) {
+                pin_loaded(bw[set][p][0]);
+                pin_loaded(bw[set][p][1]);
+                pin_loaded(sc_raw[set][p]);
+                const float sn = scale_value(sc_raw[set][p]);
+                f[p] = gi == 0 ? 1.f : s_cur[p] * __builtin_amdgcn_rcpf(sn);
+                s_cur[p] = sn;
+            }
+            // offset tile of the group: -136 * (sum of the group's activations) per row, the same in
+            // every column
+            f32x16 off[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) off[rb][r] = 0.f;
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    off[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[rb][s]), minus_bias,
+                                                                      off[rb], 0, 0, 0);
+            // into this group's units (accumulator = sum so far / scale of this group), plus the offset
+#pragma unroll
+            for (int p = 0; p < TP; ++p)
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[p][rb][r] = gi == 0 ? off[rb][r] : __builtin_fmaf(acc[p][rb][r], f[p], off[rb][r]);
+#pragma unroll
+            for (int s = 0; s < 8; ++s)
+#pragma unroll
+                for (int p = 0; p < TP; ++p) {
+                    const u32x4 &w4 = bw[set][p][s & 1];
+                    const uint32_t word = (s >> 1) == 0 ? w4.x : (s >> 1) == 1 ? w4.y : (s >> 1) == 2 ? w4.z : w4.w;
+                    const bf16x8 bexp = codes_to_bf16x8(word, dq);
+#pragma unroll
+                    for (int rb = 0; rb < 2; ++rb)
+                        acc[p][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[rb][s]), bexp,
+                                                                             acc[p][rb], 0, 0, 0);
+                }
+        });
+        // out of the last group's units
+#pragma unroll
+        for (int p = 0; p < TP; ++p)
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) acc[p][rb][r] *= s_cur[p];
+    };
+    if (full) run(std::integral_constant<int, GPW>{});
+    else if constexpr (GPW > 1) run(std::integral_constant<int, GPW - 1>{});
+
+    // --- the wavefronts' partial tiles meet in LDS: every wavefront writes its own slot (item =
+    // (pair, row block, register quad q): rows 32 rb + 8 q + 4 h ... + 3 of column l32), then item i
+    // is summed over the wavefronts, in wavefront (= ascending K) order, by wavefront i % nw
+    constexpr int kItems = TP * 2 * 4;
+    f32x4 *mine = reinterpret_cast<f32x4 *>(slot);
+#pragma unroll
+    for (int p = 0; p < TP; ++p)
+#pragma unroll
+        for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                mine[((p * 2 + rb) * 4 + q) * 64 + lane] =
+                    f32x4{acc[p][rb][4 * q], acc[p][rb][4 * q + 1], acc[p][rb][4 * q + 2], acc[p][rb][4 * q + 3]};
+    __syncthreads();
+
+    auto store_item = [&](f32x4 v, int item) {
+        const int q = item & 3, rb = (item >> 2) & 1, p = item >> 3;
+        const int row0 = 32 * rb + 8 * q + 4 * h;
+        uint16_t *dst = C + (size_t)row0 * N + (tf + 2 * p) * kTileN + l32;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (row0 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+    };
+    float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + blockIdx.x) * (kItems * 256);
+    const size_t slice_stride = (size_t)gridDim.x * (kItems * 256);  // floats between two K slices of a block
+    for (int item = wave; item < kItems; item += nw) {
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int wv = 0; wv < nw; ++wv)
+            sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[item * 64 + lane];
+        if (KS == 1) {
+            store_item(sum, item);
+        } else {
+            float *dst = partial + ks * slice_stride + item * 256 + lane * 4;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) __hip_atomic_store(dst + i, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+    if (KS == 1) return;
+
+    // Exchange between the K slices of the block's tiles: device-scope stores, acknowledged
+    // (vmcnt(0)) before the barrier that precedes the arrival count; the last block to arrive
+    // adds the slices in ascending K order and leaves the counter zero.
+    wait_vector_loads<0>();
+    __syncthreads();
+    int *counter = counters_all + blockIdx.z * gridDim.x + blockIdx.x;
+    if (tid == 0) {
+        const bool last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KS - 1;
+        s_last = last;
+        if (last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int item = wave; item < kItems; item += nw) {
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int s2 = 0; s2 < KS; ++s2) {
+            const float *src = partial + s2 * slice_stride + item * 256 + lane * 4;
+            f32x4 v;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) v[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            sum += v;
+        }
+        store_item(sum, item);
+    }
+}
+
+template <int TP, int GPW>
+hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
+    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW>>(kMidWaves * kMidSlotBytes);
+    if (attr != hipSuccess) return attr;
+    const int NT = a.N / kTileN;
+    const int runs = (a.M + kMidRows - 1) / kMidRows;
+    const int full_waves = a.GS - a.waves * (GPW - 1);
+    w4a16_mid_kernel<TP, GPW><<<dim3(NT / (2 * TP), a.KS, runs), a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
+        (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
+        a.N, a.K, a.Gs, a.KS, a.GS, full_waves);
+    return hipGetLastError();
+}
+
+template <int TP>
+hipError_t launch_mid_t(const MidArgs &a, int gpw, hipStream_t stream) {
+    switch (gpw) {
+        case 1: return launch_mid_tg<TP, 1>(a, stream);
+        case 2: return launch_mid_tg<TP, 2>(a, stream);
+        case 3: return launch_mid_tg<TP, 3>(a, stream);
+        case 4: return launch_mid_tg<TP, 4>(a, stream);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+}  // namespace
+
+int mid_max_rows_per_run() { return kMidRows; }
+
+// What a launch of the mid-M kernel assumes: whole pairs of tiles per block (N % 256 == 0 makes
+// the tile count a multiple of 16, so 2 and 4 tiles per block divide it), equal K slices, at
+// most eight wavefronts of one to four groups each, every wavefront at least one group.
+bool mid_plan_ok(const MidArgs &a) {
+    if (a.M < 1 || a.N < 256 || a.N % 256 != 0 || a.K < kGroupK || a.K % kGroupK != 0) return false;
+    if (a.pairs != 1 && a.pairs != 2) return false;
+    const int G = a.K / kGroupK;
+    if (a.KS < 1 || a.GS < 1 || a.KS * a.GS != G) return false;
+    if (a.waves < 1 || a.waves > kMidWaves || a.waves > a.GS) return false;
+    const int gpw = (a.GS + a.waves - 1) / a.waves;
+    if (gpw > kMidMaxGroups) return false;
+    const int full_waves = a.GS - a.waves * (gpw - 1);
+    return full_waves >= 1 && full_waves <= a.waves;
+}
+
+size_t mid_partial_bytes(const MidArgs &a) {
+    if (a.KS <= 1) return 0;
+    const int runs = (a.M + kMidRows - 1) / kMidRows;
+    return (size_t)runs * a.KS * (size_t)a.N * kMidRows * sizeof(float);
+}
+
+hipError_t launch_mid(const MidArgs &a, hipStream_t stream) {
+    if (!mid_plan_ok(a)) return hipErrorInvalidValue;
+    if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
+    const int gpw = (a.GS + a.waves - 1) / a.waves;
+    return a.pairs == 1 ? launch_mid_t<1>(a, gpw, stream) : launch_mid_t<2>(a, gpw, stream);
+}
+
+}  // namespace kiln
