@@ -71,13 +71,14 @@ struct MidArgs {
     const void *S;      // fp16 scales, tile layout
     void *C;            // bf16 [M, N]
     float *partial;     // mid_partial_bytes() bytes when KS > 1
-    int *counters;      // runs * N / (32 * pairs) arrival counters, zero on entry and on exit
+    int *counters;      // runs * mid_column_blocks() arrival counters, zero on entry and on exit
     int M, N, K, Gs;
     int KS;             // K slices, all of GS groups
     int GS;             // 128-row groups per slice
     int waves;          // wavefronts per block, <= 8 and <= GS; each owns ceil(GS / waves) groups or one fewer
-    int pairs;          // pairs of 16-column tiles per block: 1 or 2
+    int pairs;          // pairs of 16-column tiles per block: 1, 2 or 3
 };
+int mid_column_blocks(const MidArgs &a);
 int mid_max_rows_per_run();
 bool mid_plan_ok(const MidArgs &a);
 size_t mid_partial_bytes(const MidArgs &a);

@@ -341,19 +341,25 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
     gp->pf = p;
 }
 
-// Rows the mid-M kernel takes on the automatic plan: above the two-slab small-M instance's 32 and
-// up to two runs of 64.
-constexpr int kMidMinM = 33, kMidMaxM = 128;
+// Rows the mid-M kernel takes on the automatic plan: above the two-slab small-M instance's 32
+// (up to 32 rows that instance is ahead on every projection shape: 8.5 / 8.4 / 11.3 / 11.6 us
+// against 9.1 / 10.8 / 14.1 / 14.1) and up to two runs of 64 -- three for outputs of up to 8192
+// columns, where it still leads the matrix-core kernel's 64-row blocks at 192 rows (21.3 against
+// 23.8 us on the in-projection, 12.0 against 21.0 on the out-projection) while the widest
+// projection does not (38.8 against 34.5).
+constexpr int kMidMinM = 33, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN = 8192;
 
 // Plan for the mid-M kernel: pairs of tiles per block, K slices, wavefronts.  Cost in microseconds,
-// from the kernel's arithmetic: a wavefront issues 16 products per pair and 16 for the offset tile
-// per group, 32 cycles each at about 2.3 GHz, two wavefronts per SIMD above four per block; a
-// round of blocks costs about 1 us beside its products (first loads, reduction), an exchange
-// between K slices 2.2 us plus 0.1 us per slice.
+// fitted to a sweep of the four projection shapes at 33...192 rows: a wavefront's group step is
+// bound by the round trip of its activations through L2 and by the products of its pairs
+// (0.75 + 0.55 us per pair; every block re-reads its rows of A, so fewer and wider blocks trade
+// parallelism for L2 traffic); a launch costs about 4.5 us beside its rounds of blocks, an exchange
+// between K slices 1.5 us at two slices and 1.7 us more per further slice (out-projection at 64
+// rows: 11.5 us unsliced, 10.4 in two slices, 13.8 in four).
 MidPlan plan_mid(int m, int n, int k, int cus) {
     MidPlan best;
-    const int G = k / kGroupK, NT = n / kTileN, runs = ceil_div(m, mid_max_rows_per_run());
-    for (int pairs = 1; pairs <= 2; ++pairs) {
+    const int G = k / kGroupK, runs = ceil_div(m, mid_max_rows_per_run());
+    for (int pairs = 1; pairs <= 3; ++pairs) {
         if (g_tune.mid_pairs && pairs != g_tune.mid_pairs) continue;
         for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
             if (G % ks != 0 || (g_tune.mid_ks && ks != g_tune.mid_ks)) continue;
@@ -366,11 +372,10 @@ MidPlan plan_mid(int m, int n, int k, int cus) {
             a.waves = a.GS < 8 ? a.GS : 8;
             a.pairs = pairs;
             if (!mid_plan_ok(a)) continue;
-            const int col_blocks = NT / (2 * pairs);
+            const int col_blocks = mid_column_blocks(a);
             if ((size_t)runs * col_blocks * sizeof(int) > kCounterBytes) continue;
             const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
-            const float t_block = (float)ceil_div(a.waves, 4) * gpw * (pairs + 1) * 0.2226f;
-            const float cost = rounds * (t_block + 1.0f) + (ks > 1 ? 2.2f + 0.1f * ks : 0.f);
+            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + (ks > 1 ? 1.7f * ks - 1.9f : 0.f);
             if (!best.ok || cost < best.cost) {
                 best.ok = true;
                 best.KS = ks;
@@ -400,7 +405,8 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, bool lo
     *gp = GemmPlan{};
     // 33...128 rows of a plain GEMM: the mid-M kernel, one pass over the weights per 64 rows
     if (!lora && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
-        (g_tune.mid == 1 || (g_tune.prefill_min_m == 0 && m >= kMidMinM && m <= kMidMaxM))) {
+        (g_tune.mid == 1 ||
+         (g_tune.prefill_min_m == 0 && m >= kMidMinM && m <= (n <= kMidNarrowN ? kMidMaxMNarrow : kMidMaxM)))) {
         const MidPlan mp = plan_mid(m, n, k, cus);
         if (mp.ok) {
             gp->mid = true;
@@ -556,7 +562,7 @@ size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thre
             if (need > most) most = need;
         }
     };
-    const int small = g_tune.prefill_min_m > 128 ? g_tune.prefill_min_m : 128;
+    const int small = g_tune.prefill_min_m > kMidMaxMNarrow ? g_tune.prefill_min_m : kMidMaxMNarrow;
     for (int mm = 1; mm <= m && mm <= small; ++mm) consider(mm);
     for (int mm = 64; mm < m; mm += 64) consider(mm);
     consider(m);

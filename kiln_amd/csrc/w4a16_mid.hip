@@ -20,9 +20,10 @@
 //   * B: 2 x 128-bit per lane, pair and group, straight into the product's operand layout,
 //     requested one or two groups ahead (as the registers allow) into rotating register sets.
 //   * Scales in f32 by a running rescale of the accumulators (as in the prefill kernel); the
-//     B operand carries 136 + d, and the surplus is removed by an offset tile per group and row
-//     block (eight products with a constant -136 operand, shared by all pairs) that enters the
-//     rescale as the addend of one fused multiply-add per accumulator register.
+//     B operand carries 136 + d, and the surplus 136 * sum(a) * scale is removed after the
+//     wavefront's last group by a short extra contraction (as in the prefill kernel) over the
+//     groups' row sums, which the vector unit forms from the fragments (v_dot2c_f32_bf16) while
+//     the matrix unit multiplies.
 // At the end the wavefronts' f32 tiles are summed through LDS in wavefront (= ascending K)
 // order; K slices of a tile meet in the workspace, last arriver adds in slice order.
 #include "async_loads.h"
@@ -130,7 +131,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     // --- B: pair p = tiles tf + 2 p, tf + 2 p + 1.  Lane (l32, h) holds column l32 of the pair and
     // rows 16 s + 8 h ... + 7 of step s: word s / 2 of the 128-bit unit c + 16 (2 (s % 2) + h) of
     // chunk l32 / 16 (c = l32 % 16).  Load v = s % 2 therefore serves steps v, v + 2, v + 4, v + 6.
-    constexpr int D = TP == 1 ? 2 : 1;  // groups of look-ahead (two pairs: the registers allow one)
+    constexpr int D = TP == 1 ? 2 : 1;  // groups of look-ahead (more pairs: the registers allow one)
     constexpr int kSets = D + 1;
     u32x4 bw[kSets][TP][2];
     uint32_t sc_raw[kSets][TP];
@@ -141,10 +142,11 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         const int g = g0 + gi;
         unrolled<0, TP>([&](auto pc) {
             constexpr int p = decltype(pc)::value;
-            const char *bb = reinterpret_cast<const char *>(B) + ((size_t)(tf + 2 * p) * G + g) * 1024;
+            const int tp = min(tf + 2 * p, N / kTileN - 2);  // a pair past the last tile reads the last pair; never stored
+            const char *bb = reinterpret_cast<const char *>(B) + ((size_t)tp * G + g) * 1024;
             load_b128_streaming(bw[set][p][0], bb, b_lane);
             load_b128_streaming(bw[set][p][1], bb, b_lane + 512u);
-            const char *sb = reinterpret_cast<const char *>(S) + ((size_t)(tf + 2 * p) * Gs + (g & gs_mask)) * (kTileN * 2);
+            const char *sb = reinterpret_cast<const char *>(S) + ((size_t)tp * Gs + (g & gs_mask)) * (kTileN * 2);
             load_u16(sc_raw[set][p], sb, s_lane);
         });
     };
@@ -156,7 +158,6 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         return sv == 0.f ? 0x1p-40f : sv;
     };
 
-    const bf16x8 minus_bias = bf16x8_splat(0xC308C308u);  // bf16(-136) pairs
     const DequantConsts dq = dequant_consts();
     f32x16 acc[TP][2];
 #pragma unroll
@@ -176,6 +177,10 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         request_a(0);
         unrolled<0, (D < NG ? D : NG)>(request_b);
         float s_cur[TP];
+        float s_of[NG][TP];   // the scale of every group (this lane's column of each pair)
+        float c_of[NG][2];    // -136 * (sum of the group's activations) of row 32 rb + l32
+        uint32_t ones;
+        asm("s_mov_b32 %0, 0x3f803f80" : "=s"(ones));  // bf16 (1, 1)
         unrolled<0, NG>([&](auto gc) {
             constexpr int gi = decltype(gc)::value, set = gi % kSets;
             // this group's rows of A are in LDS; their fragments go to registers: lane (l32, h) holds
@@ -191,38 +196,47 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             wait_lds_reads();  // the slot is free again
             if constexpr (gi + 1 < NG) request_a(gi + 1);
             if constexpr (gi + D < NG) request_b(std::integral_constant<int, gi + D>{});
+            // Row sums of the group for the offset term, on the vector unit while the matrix unit
+            // multiplies: v_dot2c_f32_bf16 adds both halves of a register to an f32 sum (products with
+            // 1.0 are exact), two interleaved sums per row block; the lane's half of K here, the other
+            // half from lane + 32.
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                float e0 = 0.f, e1 = 0.f;
+#pragma unroll
+                for (int s = 0; s < 7; ++s) {
+                    asm("v_dot2c_f32_bf16 %0, %2, %1" : "+v"(e0) : "v"(af[rb][s].x), "s"(ones));
+                    asm("v_dot2c_f32_bf16 %0, %2, %1" : "+v"(e1) : "v"(af[rb][s].y), "s"(ones));
+                    asm("v_dot2c_f32_bf16 %0, %2, %1" : "+v"(e0) : "v"(af[rb][s].z), "s"(ones));
+                    asm("v_dot2c_f32_bf16 %0, %2, %1" : "+v"(e1) : "v"(af[rb][s].w), "s"(ones));
+                }
+                asm("v_dot2c_f32_bf16 %0, %2, %1" : "+v"(e0) : "v"(af[rb][7].x), "s"(ones));
+                asm("v_dot2c_f32_bf16 %0, %2, %1" : "+v"(e1) : "v"(af[rb][7].y), "s"(ones));
+                // A dot instruction may feed its own kind as the addend back to back, but another
+                // vector instruction must wait three states before it reads the result; the compiler
+                // does not know what the asm holds, so the last link of each chain carries the wait.
+                asm("v_dot2c_f32_bf16 %0, %2, %1\n\ts_nop 3" : "+v"(e0) : "v"(af[rb][7].z), "s"(ones));
+                asm("v_dot2c_f32_bf16 %0, %2, %1\n\ts_nop 3" : "+v"(e1) : "v"(af[rb][7].w), "s"(ones));
+                const float half_sum = e0 + e1;
+                c_of[gi][rb] = -kCodeBias * (half_sum + __shfl_xor(half_sum, 32, 64));
+            }
             wait_vector_loads<Sch::value.wait_b[gi]>();
-            float f[TP];
 #pragma unroll
             for (int p = 0; p < TP; ++p) {
                 pin_loaded(bw[set][p][0]);
                 pin_loaded(bw[set][p][1]);
                 pin_loaded(sc_raw[set][p]);
                 const float sn = scale_value(sc_raw[set][p]);
-                f[p] = gi == 0 ? 1.f : s_cur[p] * __builtin_amdgcn_rcpf(sn);
+                s_of[gi][p] = sn;
+                if constexpr (gi > 0) {  // into this group's units: accumulator = sum so far / scale of this group
+                    const float f = s_cur[p] * __builtin_amdgcn_rcpf(sn);
+#pragma unroll
+                    for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) acc[p][rb][r] *= f;
+                }
                 s_cur[p] = sn;
             }
-            // offset tile of the group: -136 * (sum of the group's activations) per row, the same in
-            // every column
-            f32x16 off[2];
-#pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-                for (int r = 0; r < 16; ++r) off[rb][r] = 0.f;
-#pragma unroll
-            for (int s = 0; s < 8; ++s)
-#pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
-                    off[rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[rb][s]), minus_bias,
-                                                                      off[rb], 0, 0, 0);
-            // into this group's units (accumulator = sum so far / scale of this group), plus the offset
-#pragma unroll
-            for (int p = 0; p < TP; ++p)
-#pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-                    for (int r = 0; r < 16; ++r)
-                        acc[p][rb][r] = gi == 0 ? off[rb][r] : __builtin_fmaf(acc[p][rb][r], f[p], off[rb][r]);
 #pragma unroll
             for (int s = 0; s < 8; ++s)
 #pragma unroll
@@ -243,28 +257,53 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             for (int rb = 0; rb < 2; ++rb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[p][rb][r] *= s_cur[p];
+        // The B operand carried 136 + d: remove 136 * sum(a) * scale per group by a short extra
+        // contraction.  Step e covers group 2 e in lanes 0-31 and group 2 e + 1 in lanes 32-63 (the
+        // two halves of a product's K); c is split exactly into three bf16 terms, the scale into two,
+        // and the six exact products per group add up to c * scale in the f32 accumulator.
+        unrolled<0, (NG + 1) / 2>([&](auto ec) {
+            constexpr int e = decltype(ec)::value;
+            constexpr bool has_odd = 2 * e + 1 < NG;
+            constexpr int g_odd = has_odd ? 2 * e + 1 : 2 * e;
+            bf16x8 ax[2];
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb) {
+                const float c = h ? (has_odd ? c_of[g_odd][rb] : 0.f) : c_of[2 * e][rb];
+                const uint32_t hi = __builtin_bit_cast(uint32_t, c) & 0xFFFF0000u;
+                const float r1 = c - __builtin_bit_cast(float, hi);                     // exact
+                const uint32_t mid = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
+                const float r2 = r1 - __builtin_bit_cast(float, mid);                   // exact, <= 8 significant bits
+                const uint32_t lo = __builtin_bit_cast(uint32_t, r2) & 0xFFFF0000u;
+                const u32x4 r = {(hi >> 16) | hi, (mid >> 16) | mid, (lo >> 16) | lo, 0u};
+                ax[rb] = __builtin_bit_cast(bf16x8, r);
+            }
+#pragma unroll
+            for (int p = 0; p < TP; ++p) {
+                const float sv = h ? (has_odd ? s_of[g_odd][p] : 0.f) : s_of[2 * e][p];
+                const uint32_t hi = __builtin_bit_cast(uint32_t, sv) & 0xFFFF0000u;
+                const float lo_f = sv - __builtin_bit_cast(float, hi);  // exact: f16 has 11 significant bits
+                const uint32_t pair = (hi >> 16) | (__builtin_bit_cast(uint32_t, lo_f) & 0xFFFF0000u);
+                const u32x4 r = {pair, pair, pair, 0u};
+                const bf16x8 bx = __builtin_bit_cast(bf16x8, r);
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb)
+                    acc[p][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ax[rb], bx, acc[p][rb], 0, 0, 0);
+            }
+        });
     };
     if (full) run(std::integral_constant<int, GPW>{});
     else if constexpr (GPW > 1) run(std::integral_constant<int, GPW - 1>{});
 
-    // --- the wavefronts' partial tiles meet in LDS: every wavefront writes its own slot (item =
-    // (pair, row block, register quad q): rows 32 rb + 8 q + 4 h ... + 3 of column l32), then item i
-    // is summed over the wavefronts, in wavefront (= ascending K) order, by wavefront i % nw
+    // --- the wavefronts' partial tiles meet in LDS, at most two pairs at a time (a wavefront's
+    // 16 KiB slot holds two pairs' tiles): every wavefront writes its own slot (item = (pair, row
+    // block, register quad q): rows 32 rb + 8 q + 4 h ... + 3 of column l32), then item i is summed
+    // over the wavefronts, in wavefront (= ascending K) order, by wavefront i % nw.
     constexpr int kItems = TP * 2 * 4;
-    f32x4 *mine = reinterpret_cast<f32x4 *>(slot);
-#pragma unroll
-    for (int p = 0; p < TP; ++p)
-#pragma unroll
-        for (int rb = 0; rb < 2; ++rb)
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-                mine[((p * 2 + rb) * 4 + q) * 64 + lane] =
-                    f32x4{acc[p][rb][4 * q], acc[p][rb][4 * q + 1], acc[p][rb][4 * q + 2], acc[p][rb][4 * q + 3]};
-    __syncthreads();
-
+    const int NT = N / kTileN;
     auto store_item = [&](f32x4 v, int item) {
         const int q = item & 3, rb = (item >> 2) & 1, p = item >> 3;
         const int row0 = 32 * rb + 8 * q + 4 * h;
+        if (tf + 2 * p >= NT) return;  // a pair past the last tile (grid padding)
         uint16_t *dst = C + (size_t)row0 * N + (tf + 2 * p) * kTileN + l32;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -272,18 +311,33 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     };
     float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + blockIdx.x) * (kItems * 256);
     const size_t slice_stride = (size_t)gridDim.x * (kItems * 256);  // floats between two K slices of a block
-    for (int item = wave; item < kItems; item += nw) {
-        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-        for (int wv = 0; wv < nw; ++wv)
-            sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[item * 64 + lane];
-        if (KS == 1) {
-            store_item(sum, item);
-        } else {
-            float *dst = partial + ks * slice_stride + item * 256 + lane * 4;
+    f32x4 *mine = reinterpret_cast<f32x4 *>(slot);
+    unrolled<0, (TP + 1) / 2>([&](auto phc) {
+        constexpr int p0 = 2 * decltype(phc)::value, p1 = p0 + 2 < TP ? p0 + 2 : TP;
+        if constexpr (p0 > 0) __syncthreads();  // the previous phase's sums have been read
 #pragma unroll
-            for (int i = 0; i < 4; ++i) __hip_atomic_store(dst + i, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        for (int p = p0; p < p1; ++p)
+#pragma unroll
+            for (int rb = 0; rb < 2; ++rb)
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    mine[(((p - p0) * 2 + rb) * 4 + q) * 64 + lane] =
+                        f32x4{acc[p][rb][4 * q], acc[p][rb][4 * q + 1], acc[p][rb][4 * q + 2], acc[p][rb][4 * q + 3]};
+        __syncthreads();
+        for (int item = p0 * 8 + wave; item < p1 * 8; item += nw) {
+            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+            for (int wv = 0; wv < nw; ++wv)
+                sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[(item - p0 * 8) * 64 + lane];
+            if (KS == 1) {
+                store_item(sum, item);
+            } else {
+                float *dst = partial + ks * slice_stride + item * 256 + lane * 4;
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    __hip_atomic_store(dst + i, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
-    }
+    });
     if (KS == 1) return;
 
     // Exchange between the K slices of the block's tiles: device-scope stores, acknowledged
@@ -319,7 +373,8 @@ hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
     const int full_waves = a.GS - a.waves * (GPW - 1);
-    w4a16_mid_kernel<TP, GPW><<<dim3(NT / (2 * TP), a.KS, runs), a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
+    w4a16_mid_kernel<TP, GPW><<<dim3((NT + 2 * TP - 1) / (2 * TP), a.KS, runs), a.waves * 64, a.waves * kMidSlotBytes,
+                               stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
         a.N, a.K, a.Gs, a.KS, a.GS, full_waves);
     return hipGetLastError();
@@ -340,32 +395,38 @@ hipError_t launch_mid_t(const MidArgs &a, int gpw, hipStream_t stream) {
 
 int mid_max_rows_per_run() { return kMidRows; }
 
-// What a launch of the mid-M kernel assumes: whole pairs of tiles per block (N % 256 == 0 makes
-// the tile count a multiple of 16, so 2 and 4 tiles per block divide it), equal K slices, at
-// most eight wavefronts of one to four groups each, every wavefront at least one group.
+// What a launch of the mid-M kernel assumes: one to three pairs of tiles per block (N % 256 == 0
+// makes the tile count even; a last block may hold fewer pairs), equal K slices, at most eight
+// wavefronts of one to four groups each, every wavefront at least one group.
 bool mid_plan_ok(const MidArgs &a) {
     if (a.M < 1 || a.N < 256 || a.N % 256 != 0 || a.K < kGroupK || a.K % kGroupK != 0) return false;
-    if (a.pairs != 1 && a.pairs != 2) return false;
+    if (a.pairs < 1 || a.pairs > 3) return false;
     const int G = a.K / kGroupK;
     if (a.KS < 1 || a.GS < 1 || a.KS * a.GS != G) return false;
     if (a.waves < 1 || a.waves > kMidWaves || a.waves > a.GS) return false;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
-    if (gpw > kMidMaxGroups) return false;
+    if (gpw > kMidMaxGroups || (a.pairs == 3 && gpw == 4)) return false;  // (3, 4) would spill registers
     const int full_waves = a.GS - a.waves * (gpw - 1);
     return full_waves >= 1 && full_waves <= a.waves;
 }
 
+int mid_column_blocks(const MidArgs &a) { return (a.N / kTileN + 2 * a.pairs - 1) / (2 * a.pairs); }
+
 size_t mid_partial_bytes(const MidArgs &a) {
     if (a.KS <= 1) return 0;
-    const int runs = (a.M + kMidRows - 1) / kMidRows;
-    return (size_t)runs * a.KS * (size_t)a.N * kMidRows * sizeof(float);
+    const int runs = (a.M + kMidRows - 1) / kMidRows, col_blocks = mid_column_blocks(a);
+    return (size_t)runs * a.KS * col_blocks * (size_t)(a.pairs * 32) * kMidRows * sizeof(float);
 }
 
 hipError_t launch_mid(const MidArgs &a, hipStream_t stream) {
     if (!mid_plan_ok(a)) return hipErrorInvalidValue;
     if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
-    return a.pairs == 1 ? launch_mid_t<1>(a, gpw, stream) : launch_mid_t<2>(a, gpw, stream);
+    switch (a.pairs) {
+        case 1: return launch_mid_t<1>(a, gpw, stream);
+        case 2: return launch_mid_t<2>(a, gpw, stream);
+        default: return launch_mid_t<3>(a, gpw, stream);
+    }
 }
 
 }  // namespace kiln
