@@ -138,14 +138,14 @@ kiln_marlin_status_t kiln_w4a16_gemm_lora(
 
 /*
  * C[m, n_out] = silu(gate) * up with [gate | up] = A * dequant(B, s), the fused MLP
- * input projection followed by SwiGLU in one call.  The reference issues gate and up
- * as two GEMMs and then silu and a multiply as separate kernels on bf16 tensors
- * (crates/kiln-model/src/forward.rs:2771-2819); here the product is formed from the
- * f32 accumulators (M >= 33) and rounded once.
- *   B, s   packed for 2 * n_out columns by kiln_w4a16_interleave_gate_up (per 64
- *          packed columns: 32 gate columns, then the 32 matching up columns);
- *          n_out % 128 == 0.
- *   workspace: kiln_w4a16_swiglu_workspace_bytes(m, n_out, k) bytes, zero on first use.
+ * input projection followed by SwiGLU in one call, at any m.  The reference issues gate and
+ * up as two GEMMs and then silu and a multiply as separate kernels on bf16 tensors
+ * (crates/kiln-model/src/forward.rs:2771-2819); here every kernel forms the product from its
+ * f32 sums where it stores a tile and rounds once: one launch, no intermediate tensor.
+ *   B, s   packed for 2 * n_out columns by kiln_w4a16_interleave_gate_up (per 16 packed
+ *          columns: 8 gate columns, then the 8 matching up columns); n_out % 128 == 0.
+ *   workspace: kiln_w4a16_swiglu_workspace_bytes(m, n_out, k) bytes (= the plain GEMM's for
+ *          2 * n_out columns), counter prefix zero on first use.
  */
 kiln_marlin_status_t kiln_w4a16_gemm_swiglu(
     const void *A, const void *B, void *C, const void *s,
@@ -192,8 +192,8 @@ kiln_marlin_status_t kiln_w4a16_unpack_to_gptq(
 
 /*
  * Interleave two packed projections of equal shape [k, n_each] (gate, up) into the
- * packed form kiln_w4a16_gemm_swiglu reads: [k, 2 * n_each] with, per 64 columns,
- * 32 gate columns then the 32 matching up columns.  n_each % 128 == 0.
+ * packed form kiln_w4a16_gemm_swiglu reads: [k, 2 * n_each] with, per 16 columns (one
+ * column tile), 8 gate columns then the 8 matching up columns.  n_each % 128 == 0.
  * No counterpart in the reference (its gate and up stay separate tensors).
  */
 kiln_marlin_status_t kiln_w4a16_interleave_gate_up(

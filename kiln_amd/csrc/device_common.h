@@ -70,6 +70,43 @@ __device__ __forceinline__ bf16x8 bf16x8_splat(uint32_t pair) {
     return __builtin_bit_cast(bf16x8, r);
 }
 
+// Store four rows (row0 ... row0 + 3, those below M) of column c of 16-column tile tt from a lane
+// of the 16x16 accumulator layout (lane = c + 16 q holds rows 4 q ... 4 q + 3 of column c).
+// swiglu: the tile holds 8 gate columns, then the 8 matching up columns (the packing of
+// kiln_w4a16_interleave_gate_up); the lane of gate column c takes up from lane c + 8 of its
+// 16-lane row and stores silu(gate) * up = gate / (1 + exp(-gate)) * up into a result half as wide
+// (crates/kiln-model/src/forward.rs:2789-2819 forms it from bf16 tensors; here from the f32 sums,
+// rounded once).  Every lane of the wavefront must be active.
+__device__ __forceinline__ void store_tile_rows(uint16_t *__restrict__ C, int N, int M, int row0, int tt, int c,
+                                                f32x4 v, bool swiglu) {
+    if (!swiglu) {
+        uint16_t *dst = C + (size_t)row0 * N + tt * kTileN + c;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (row0 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+        return;
+    }
+    const int n_out = N >> 1;
+    f32x4 up;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {  // row_ror:8 inside each row of 16 lanes
+        const float vi = v[i];  // a scalar copy: bit-casting the vector element in place reads element 0
+            up[i] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, vi), 0x128, 0xF, 0xF, true));
+        // the exchange must run while all lanes are active: keep it from being folded into the
+        // arithmetic below, which runs for the gate lanes only (a disabled source lane reads as zero)
+        asm volatile("" : "+v"(up[i]));
+    }
+    if ((c & 8) == 0) {
+        uint16_t *dst = C + (size_t)row0 * n_out + tt * (kTileN / 2) + c;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (row0 + i < M) {
+                const float gate = v[i];
+                dst[(size_t)i * n_out] = f32_to_bf16_bits(gate * __builtin_amdgcn_rcpf(1.f + __expf(-gate)) * up[i]);
+            }
+    }
+}
+
 __device__ __forceinline__ bf16x8 bf16x8_zero() {
     u32x4 r = {0u, 0u, 0u, 0u};
     return __builtin_bit_cast(bf16x8, r);

@@ -34,6 +34,7 @@ struct DecodeArgs {
     int r_total = 0;               // <= 64
     int lora_slices = 1;
     int lora_rows = 0;             // rows of the whole projection (>= M: the slab may be a part of it)
+    bool swiglu = false;  // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
     int group_major = -1; // tuning: 0 never a group-major instance, 1 only the LDS-staged one, 2 the
                           // register-fragment one wherever a plan fits it; -1: automatic
 };
@@ -77,6 +78,7 @@ struct MidArgs {
     int GS;             // 128-row groups per slice
     int waves;          // wavefronts per block, <= 8 and <= GS; each owns ceil(GS / waves) groups or one fewer
     int pairs;          // pairs of 16-column tiles per block: 1, 2 or 3
+    bool swiglu;        // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
 };
 int mid_column_blocks(const MidArgs &a);
 int mid_max_rows_per_run();
@@ -104,7 +106,7 @@ struct PrefillArgs {
     int KS = 1;
     int bn = 128;                   // block columns: 128 or 256
     int bm = 256;                   // block rows: 64, 128 or 256
-    bool swiglu = false;            // columns are gate/up interleaved by 32; C is [M, N/2] = silu(gate) * up
+    bool swiglu = false;            // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
     int nb_full = 0;                // leading column blocks computed as whole tiles; the rest is sliced
     int cus = 256;                  // compute units of the device
     float *partial = nullptr;       // prefill_partial_bytes(M, N, KS) bytes

@@ -236,21 +236,28 @@ kiln_marlin_status_t kiln_w4a16_interleave_gate_up(const int32_t *gate_b, const 
                                                    const int32_t *up_b, const uint16_t *up_s, int k, int n_each,
                                                    int groupsize, int32_t *out_b, uint16_t *out_s) {
     if (!gate_b || !gate_s || !up_b || !up_s || !out_b || !out_s) return KILN_W4A16_ERR_ARGUMENT;
-    // 32 columns = two column tiles at a time; the fused width 2 * n_each must itself be a legal width
+    // the fused width 2 * n_each must itself be a legal width
     if (n_each <= 0 || n_each % 128 != 0 || !shape_ok(k, 2 * n_each, groupsize)) return KILN_W4A16_ERR_PROB_SHAPE;
     const int G = k / kGroupK;
     const int Gs = (groupsize == -1) ? 1 : G;
     const size_t tile_words = (size_t)G * kChunkWords, tile_scales = (size_t)Gs * kTileN;
-    parallel_for(n_each / 32, [&](int j) {
+    // Output tile j = gate columns 8 j ... 8 j + 7, then up columns 8 j ... 8 j + 7: half of source
+    // tile j / 2.  In a chunk, lane c + 16 kq owns four words, so the eight lanes of a half tile and
+    // one kq are 128 contiguous bytes on both sides.
+    parallel_for(n_each / 8, [&](int j) {
+        const size_t src_tile = (size_t)j / 2;
+        const int c0 = 8 * (j & 1);  // first source column inside its tile
         for (int half = 0; half < 2; ++half) {  // gate, then up
-            const int32_t *src_b = half ? up_b : gate_b;
-            const uint16_t *src_s = half ? up_s : gate_s;
-            for (int t = 0; t < 2; ++t) {
-                const size_t src_tile = (size_t)2 * j + t, dst_tile = (size_t)4 * j + 2 * half + t;
-                std::memcpy(out_b + dst_tile * tile_words, src_b + src_tile * tile_words, tile_words * sizeof(int32_t));
-                std::memcpy(out_s + dst_tile * tile_scales, src_s + src_tile * tile_scales,
-                            tile_scales * sizeof(uint16_t));
-            }
+            const int32_t *src_b = (half ? up_b : gate_b) + src_tile * tile_words;
+            const uint16_t *src_s = (half ? up_s : gate_s) + src_tile * tile_scales;
+            int32_t *dst_b = out_b + (size_t)j * tile_words;
+            uint16_t *dst_s = out_s + (size_t)j * tile_scales;
+            for (int g = 0; g < G; ++g)
+                for (int kq = 0; kq < 4; ++kq)
+                    std::memcpy(dst_b + (size_t)g * kChunkWords + (size_t)(8 * half + 16 * kq) * 4,
+                                src_b + (size_t)g * kChunkWords + (size_t)(c0 + 16 * kq) * 4, 8 * 4 * sizeof(int32_t));
+            for (int gs = 0; gs < Gs; ++gs)
+                std::memcpy(dst_s + (size_t)gs * kTileN + 8 * half, src_s + (size_t)gs * kTileN + c0, 8 * sizeof(uint16_t));
         }
     });
     return KILN_W4A16_OK;

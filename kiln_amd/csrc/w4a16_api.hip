@@ -511,35 +511,6 @@ using namespace kiln;
 namespace kiln {
 namespace {
 
-// out[row][32 b + i] = silu(t[row][64 b + i]) * t[row][64 b + 32 + i] for the gate/up-by-32
-// interleaved GEMM result t (bf16, [m, 2 n_out]); one thread per 8 output columns.
-__global__ __launch_bounds__(256) void swiglu_rows_kernel(const uint16_t *__restrict__ t, uint16_t *__restrict__ out,
-                                                        int m, int n_out) {
-    const int item = blockIdx.x * 256 + threadIdx.x;
-    const int per_row = n_out / 8;
-    if (item >= m * per_row) return;
-    const int row = item / per_row, j8 = (item - row * per_row) * 8;  // first of 8 output columns
-    const uint16_t *src = t + (size_t)row * 2 * n_out + (j8 / 32) * 64 + (j8 % 32);
-    const u32x4 g4 = *reinterpret_cast<const u32x4 *>(src), u4 = *reinterpret_cast<const u32x4 *>(src + 32);
-    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
-    uint32_t ow[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const float g0 = __builtin_bit_cast(float, gw[i] << 16), g1 = __builtin_bit_cast(float, gw[i] & 0xFFFF0000u);
-        const float u0 = __builtin_bit_cast(float, uw[i] << 16), u1 = __builtin_bit_cast(float, uw[i] & 0xFFFF0000u);
-        const float h0 = g0 * __builtin_amdgcn_rcpf(1.f + __expf(-g0)) * u0;
-        const float h1 = g1 * __builtin_amdgcn_rcpf(1.f + __expf(-g1)) * u1;
-        ow[i] = (uint32_t)f32_to_bf16_bits(h0) | ((uint32_t)f32_to_bf16_bits(h1) << 16);
-    }
-    *reinterpret_cast<u32x4 *>(out + (size_t)row * n_out + j8) = u32x4{ow[0], ow[1], ow[2], ow[3]};
-}
-
-}  // namespace
-}  // namespace kiln
-
-namespace kiln {
-namespace {
-
 struct LoraSpec {
     const void *a;       // bf16 [r_total, K]
     const void *b;       // bf16 [N, r_total]
@@ -573,7 +544,7 @@ size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thre
 // optional low-rank term.
 kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void *s, int prob_m, int prob_n,
                               int prob_k, void *workspace, int groupsize, int dev, void *stream, int thread_k,
-                              int thread_n, int sms, const LoraSpec *lora) {
+                              int thread_n, int sms, const LoraSpec *lora, bool swiglu = false) {
     if (prob_m < 0 || prob_n < 0 || prob_k < 0) return KILN_W4A16_ERR_PROB_SHAPE;
     if (!shape_ok(prob_n, prob_k, groupsize)) return KILN_W4A16_ERR_PROB_SHAPE;
     if (thread_k > 0 && thread_k % 128 != 0) return KILN_W4A16_ERR_PROB_SHAPE;
@@ -608,6 +579,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             pa.ranks = lora->ranks;
             pa.scales = lora->scales;
         }
+        pa.swiglu = swiglu;
         pa.cus = cus;
         pa.KS = gp.pf.ks;
         pa.bn = gp.pf.bn;
@@ -625,6 +597,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         ma.S = s;
         ma.C = C;
         ma.Gs = (groupsize == -1) ? 1 : prob_k / kGroupK;
+        ma.swiglu = swiglu;
         ma.counters = reinterpret_cast<int *>(workspace);
         ma.partial = reinterpret_cast<float *>(ws + wl.decode_partial);
         return launch_mid(ma, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
@@ -653,10 +626,12 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     a.N = prob_n;
     a.K = prob_k;
     a.Gs = (groupsize == -1) ? 1 : prob_k / kGroupK;
+    a.swiglu = swiglu;
+    const int ldc = swiglu ? prob_n / 2 : prob_n;  // the fused gate/up result is half as wide
     for (int i = 0; i < gp.launches; ++i) {
         const DecodeLaunch &l = gp.dl[i];
         a.A = reinterpret_cast<const uint16_t *>(A) + (size_t)l.r0 * prob_k;
-        a.C = reinterpret_cast<uint16_t *>(C) + (size_t)l.r0 * prob_n;
+        a.C = reinterpret_cast<uint16_t *>(C) + (size_t)l.r0 * ldc;
         if (lora) {
             a.lora_t = reinterpret_cast<const uint16_t *>(lora_t) + (size_t)l.r0 * rp;
             a.lora_b = lora->b;
@@ -860,73 +835,18 @@ kiln_marlin_status_t kiln_w4a16_gemm_lora(const void *A, const void *B, void *C,
     return gemm_any(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream, -1, -1, -1, &lora);
 }
 
-static size_t swiglu_tmp_offset(int m, int n, int k) {
-    return (kiln_w4a16_workspace_bytes(m, n, k) + 255) & ~(size_t)255;
-}
-
 kiln_marlin_status_t kiln_w4a16_gemm_swiglu(const void *A, const void *B, void *C, const void *s,
                                             int prob_m, int n_out, int prob_k, void *workspace,
                                             int groupsize, int dev, void *stream) {
     if (prob_m < 0 || n_out < 0 || prob_k < 0 || n_out > INT32_MAX / 2) return KILN_W4A16_ERR_PROB_SHAPE;
-    const int prob_n = 2 * n_out;  // packed columns: gate and up interleaved by 32
-    if (!shape_ok(prob_n, prob_k, groupsize)) return KILN_W4A16_ERR_PROB_SHAPE;
-    if (prob_m == 0 || n_out == 0 || prob_k == 0) return KILN_W4A16_OK;
-    if (!A || !B || !C || !s || !workspace) return KILN_W4A16_ERR_ARGUMENT;
-    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const int cus = compute_units(dev);
-    if (prob_m <= 32 && !(g_tune.prefill_min_m > 0 && prob_m >= g_tune.prefill_min_m)) {
-        // decode regime: the GEMM as usual into scratch behind the workspace, then one
-        // elementwise pass over the few rows
-        uint16_t *tmp = reinterpret_cast<uint16_t *>(reinterpret_cast<char *>(workspace) +
-                                                     swiglu_tmp_offset(prob_m, prob_n, prob_k));
-        const kiln_marlin_status_t rc = kiln_marlin_w4a16_gemm(A, B, tmp, const_cast<void *>(s), prob_m, prob_n,
-                                                               prob_k, workspace, groupsize, dev, stream, -1, -1,
-                                                               -1, 16);
-        if (rc != KILN_W4A16_OK) return rc;
-        const int items = prob_m * (n_out / 8);
-        swiglu_rows_kernel<<<(items + 255) / 256, 256, 0, st>>>(tmp, reinterpret_cast<uint16_t *>(C), prob_m, n_out);
-        return hipGetLastError() == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
-    }
-    GemmPlan gp;
-    plan_as_prefill(prob_m, prob_n, prob_k, cus, -1, -1, &gp);
-    const WorkspaceLayout wl = workspace_layout(gp, prob_m, prob_n, prob_k);
-    PrefillArgs pa{};
-    pa.A = A;
-    pa.B = B;
-    pa.S = s;
-    pa.C = C;
-    pa.aext = reinterpret_cast<char *>(workspace) + wl.aext;
-    pa.M = prob_m;
-    pa.N = prob_n;
-    pa.K = prob_k;
-    pa.Gs = (groupsize == -1) ? 1 : prob_k / kGroupK;
-    pa.swiglu = true;
-    pa.cus = cus;
-    pa.KS = gp.pf.ks;
-    pa.bn = gp.pf.bn;
-    pa.bm = gp.pf.bm;
-    pa.nb_full = gp.pf.nb_full;
-    pa.counters = reinterpret_cast<int *>(workspace);
-    pa.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + wl.prefill_partial);
-    return launch_prefill(pa, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+    // packed columns: per 16-column tile 8 gate columns, then the 8 matching up columns; every kernel
+    // forms silu(gate) * up where it stores a tile, from the f32 sums
+    return gemm_any(A, B, C, s, prob_m, 2 * n_out, prob_k, workspace, groupsize, dev, stream, -1, -1, -1, nullptr, true);
 }
 
 size_t kiln_w4a16_swiglu_workspace_bytes(int prob_m, int n_out, int prob_k) {
-    const int m = prob_m > 0 ? prob_m : 1;
-    if (n_out <= 0 || prob_k <= 0 || !shape_ok(2 * n_out, prob_k, 128)) return kCounterBytes;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) dev = -1;
-    const int cus = compute_units(dev);
-    // the plain GEMM's need for every m' <= m (rows up to 32 run it), the matrix-core path's need for
-    // every row-block count up to m's, and room for the decode regime's [32, 2 n_out] bf16 intermediate
-    size_t most = swiglu_tmp_offset(m, 2 * n_out, prob_k) + (size_t)32 * 2 * n_out * sizeof(uint16_t);
-    for (int mm = 64; mm < m + 64; mm += 64) {
-        GemmPlan gp;
-        plan_as_prefill(mm < m ? mm : m, 2 * n_out, prob_k, cus, -1, -1, &gp);
-        const size_t need = workspace_layout(gp, mm < m ? mm : m, 2 * n_out, prob_k).total;
-        if (need > most) most = need;
-    }
-    return most;
+    if (n_out <= 0 || n_out > INT32_MAX / 2) return kCounterBytes;
+    return kiln_w4a16_workspace_bytes(prob_m, 2 * n_out, prob_k);  // the same plans as the plain GEMM of that width
 }
 
 }  // extern "C"

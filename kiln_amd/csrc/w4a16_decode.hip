@@ -167,7 +167,7 @@ template <int U, bool DIRECT, bool CROSS, bool LORA>
 __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_decode_kernel(
     const uint16_t *__restrict__ A, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C, float *partial, int *counters, int M, int N, int K, int Gs, int KS,
-    int GS, int BPS, LoraTail lo) {
+    int GS, int BPS, int swiglu, LoraTail lo) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ int s_last[kMaxTouched];
 
@@ -403,10 +403,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_decode_kernel(
     const int q4 = lane >> 4, c = lane & 15;
     auto store_tile = [&](f32x4 v, int tt) {
         if constexpr (LORA) lora_add(v, lo, 0, M, tt, lane);
-        uint16_t *dst = C + (size_t)(4 * q4) * N + tt * kTileN + c;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (4 * q4 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+        store_tile_rows(C, N, M, 4 * q4, tt, c, v, swiglu != 0);
     };
     for (int ti = wave; ti < ntouched; ti += nw) {
         const int tt = tf + ti;
@@ -491,7 +488,7 @@ template <int T, int GPW, bool LORA>
 __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_decode_gm_kernel(
     const uint16_t *__restrict__ A, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C, float *partial, int *counters, int M, int N, int K, int Gs, int KS,
-    int GS, int full_waves, LoraTail lo) {
+    int GS, int full_waves, int swiglu, LoraTail lo) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ int s_last[T];
     const int tid = threadIdx.x;
@@ -600,10 +597,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_decode_gm_kernel(
     const int q4 = lane >> 4, c = lane & 15;
     auto store_tile = [&](f32x4 v, int tt) {
         if constexpr (LORA) lora_add(v, lo, 0, M, tt, lane);
-        uint16_t *dst = C + (size_t)(4 * q4) * N + tt * kTileN + c;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (4 * q4 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+        store_tile_rows(C, N, M, 4 * q4, tt, c, v, swiglu != 0);
     };
     const int tiles = min(T, NT - tf);
     for (int ti = wave; ti < tiles; ti += nw) {
@@ -689,7 +683,7 @@ template <int T, int GPW, int SL, bool LORA>
 __global__ __launch_bounds__(12 * 64) void w4a16_decode_gmr_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
-    int GS, LoraTail lo) {
+    int GS, int swiglu, LoraTail lo) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     __shared__ int s_last[T];
     constexpr int U = T * GPW;  // chunks per wavefront
@@ -703,7 +697,7 @@ __global__ __launch_bounds__(12 * 64) void w4a16_decode_gmr_kernel(
     // tiles; a launch of several runs saves the gap between two launches, nothing else)
     const int zr = blockIdx.z * (16 * SL);
     const uint16_t *__restrict__ A = A_all + (size_t)zr * K;
-    uint16_t *__restrict__ C = C_all + (size_t)zr * N;
+    uint16_t *__restrict__ C = C_all + (size_t)zr * (swiglu ? N >> 1 : N);  // the fused result is half as wide
     float *partial = partial_all + (size_t)blockIdx.z * KS * 2 * NT * 256;
     int *counters = counters_all + blockIdx.z * NT;
     const int M = min(rows - zr, 16 * SL);
@@ -808,11 +802,7 @@ __global__ __launch_bounds__(12 * 64) void w4a16_decode_gmr_kernel(
     const int q4 = lane >> 4, c = lane & 15;
     auto store_tile = [&](f32x4 v, int tt, int sl) {
         if constexpr (LORA) lora_add(v, lo, 16 * sl, M, tt, lane);
-        const int row0 = 16 * sl + 4 * q4;
-        uint16_t *dst = C + (size_t)row0 * N + tt * kTileN + c;
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (row0 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+        store_tile_rows(C, N, M, 16 * sl + 4 * q4, tt, c, v, swiglu != 0);
     };
     const int tiles = min(T, NT - tf);
     for (int it = wave; it < tiles * SL; it += nw) {
@@ -880,7 +870,7 @@ hipError_t launch_gmr_tgs(const DecodeArgs &a, hipStream_t stream) {
     w4a16_decode_gmr_kernel<T, GPW, SL, kLora><<<dim3((NT + T - 1) / T, a.KS, runs), a.waves * 64,
                                                  decode_gmr_lds_bytes(a.waves, T, SL), stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial,
-        a.counters, a.rows > a.M ? a.rows : a.M, a.N, a.K, a.Gs, a.KS, a.GS, lora_tail(a));
+        a.counters, a.rows > a.M ? a.rows : a.M, a.N, a.K, a.Gs, a.KS, a.GS, a.swiglu ? 1 : 0, lora_tail(a));
     return hipGetLastError();
 }
 
@@ -926,7 +916,7 @@ hipError_t launch_gm_tg(const DecodeArgs &a, hipStream_t stream) {
     w4a16_decode_gm_kernel<T, GPW, kLora><<<dim3((NT + T - 1) / T, a.KS), a.waves * 64,
                                             decode_gm_lds_bytes(a.GS, a.waves, T), stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial,
-        a.counters, a.M, a.N, a.K, a.Gs, a.KS, a.GS, full_waves, lora_tail(a));
+        a.counters, a.M, a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, lora_tail(a));
     return hipGetLastError();
 }
 
@@ -948,7 +938,7 @@ hipError_t launch_udc(const DecodeArgs &a, hipStream_t stream) {
     const size_t lds = decode_lds_bytes(a.GS, a.waves, DIRECT);
     w4a16_decode_kernel<U, DIRECT, CROSS, kLora><<<dim3(a.BPS, a.KS), a.waves * 64, lds, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial,
-        a.counters, a.M, a.N, a.K, a.Gs, a.KS, a.GS, a.BPS, lora_tail(a));
+        a.counters, a.M, a.N, a.K, a.Gs, a.KS, a.GS, a.BPS, a.swiglu ? 1 : 0, lora_tail(a));
     return hipGetLastError();
 }
 
@@ -1019,6 +1009,7 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t stream) {
     const int gs_last = G - (a.KS - 1) * a.GS;  // smallest slice
     const bool sane = a.waves >= 1 && a.waves <= kMaxWaves && a.M >= 1 && a.U >= 1 && a.GS >= 1 && a.KS >= 1;
     if (a.r_total < 0 || a.r_total > 64) return hipErrorInvalidValue;
+    if (a.swiglu && a.r_total > 0) return hipErrorInvalidValue;  // the low-rank term has no gate/up split
     if (a.r_total > 0 && (!a.lora_t || !a.lora_b || a.lora_slices < 1 || a.lora_rows < a.M)) return hipErrorInvalidValue;
     if (a.rows > a.M && (!a.regs || a.M != 32 || a.rows > 128)) return hipErrorInvalidValue;  // up to four runs of 32 rows
     if (a.regs) {

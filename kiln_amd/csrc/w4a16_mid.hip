@@ -88,7 +88,7 @@ template <int TP, int GPW>
 __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
-    int GS, int full_waves) {
+    int GS, int full_waves, int swiglu) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     __shared__ int s_last;
     const int tid = threadIdx.x;
@@ -101,7 +101,8 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const int zr = blockIdx.z * kMidRows;
     const int M = min(rows - zr, kMidRows);
     const uint16_t *__restrict__ A = A_all + (size_t)zr * K;
-    uint16_t *__restrict__ C = C_all + (size_t)zr * N;
+    const int ldc = swiglu ? N >> 1 : N;  // the fused gate/up result is half as wide
+    uint16_t *__restrict__ C = C_all + (size_t)zr * ldc;
     const int ks = blockIdx.y;
     const int tf = blockIdx.x * (2 * TP);  // first 16-column tile of the block
     // the first `full_waves` wavefronts own GPW groups each, the others GPW - 1
@@ -303,11 +304,32 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     auto store_item = [&](f32x4 v, int item) {
         const int q = item & 3, rb = (item >> 2) & 1, p = item >> 3;
         const int row0 = 32 * rb + 8 * q + 4 * h;
-        if (tf + 2 * p >= NT) return;  // a pair past the last tile (grid padding)
-        uint16_t *dst = C + (size_t)row0 * N + (tf + 2 * p) * kTileN + l32;
+        const bool live = tf + 2 * p < NT;  // false: a pair past the last tile (grid padding)
+        if (!swiglu) {
+            uint16_t *dst = C + (size_t)row0 * N + (tf + 2 * p) * kTileN + l32;
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-            if (row0 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+            for (int i = 0; i < 4; ++i)
+                if (live && row0 + i < M) dst[(size_t)i * N] = f32_to_bf16_bits(v[i]);
+            return;
+        }
+        // gate/up interleaved by 8 inside every tile: the lane of gate column c takes up from lane
+        // c + 8 of its 16-lane row and stores silu(gate) * up (forward.rs:2789-2819) half as wide
+        f32x4 up;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float vi = v[i];  // a scalar copy: bit-casting the vector element in place reads element 0
+            up[i] = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, vi), 0x128, 0xF, 0xF, true));
+            asm volatile("" : "+v"(up[i]));  // exchanged while all lanes are active, not folded into the gate lanes' arithmetic
+        }
+        if (live && (l32 & 8) == 0) {
+            uint16_t *dst = C + (size_t)row0 * ldc + (tf + 2 * p) * (kTileN / 2) + (l32 >> 4) * 8 + (l32 & 7);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (row0 + i < M) {
+                    const float gate = v[i];
+                    dst[(size_t)i * ldc] = f32_to_bf16_bits(gate * __builtin_amdgcn_rcpf(1.f + __expf(-gate)) * up[i]);
+                }
+        }
     };
     float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + blockIdx.x) * (kItems * 256);
     const size_t slice_stride = (size_t)gridDim.x * (kItems * 256);  // floats between two K slices of a block
@@ -376,7 +398,7 @@ hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
     w4a16_mid_kernel<TP, GPW><<<dim3((NT + 2 * TP - 1) / (2 * TP), a.KS, runs), a.waves * 64, a.waves * kMidSlotBytes,
                                stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
-        a.N, a.K, a.Gs, a.KS, a.GS, full_waves);
+        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0);
     return hipGetLastError();
 }
 

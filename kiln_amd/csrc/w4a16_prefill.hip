@@ -320,8 +320,9 @@ __device__ __forceinline__ float dpp_move(float v) {
 // Block shape: WM x NWN wavefronts, each owning MI x 2 tiles of 32 x 32 (MI * 32 rows x 64
 // columns).  WM = 2, MI = 4: 256-row blocks (256 x 128 with 4 wavefronts, 256 x 256 with 8);
 // WM = 1: 128-row (MI = 4) and 64-row (MI = 2) blocks for small M.
-// SWIGLU: the packed columns hold, per 64, 32 gate columns then the 32 matching up columns
-// (a wavefront's two column sub-tiles); the store writes silu(gate) * up, half as wide
+// SWIGLU: every 16-column tile of the packed weight holds 8 gate columns, then the 8 matching up
+// columns; a wavefront's sub-tile 0 gathers the gate columns of its four tiles and sub-tile 1 the
+// up columns; the store writes silu(gate) * up, half as wide
 // (crates/kiln-model/src/forward.rs:2771-2819 computes gate, up, silu and the product as
 // separate bf16 tensors; here the product is formed from the f32 accumulators and rounded once).
 // RS: the row sums of A that the offset removal needs are formed inside the kernel from the A
@@ -418,10 +419,14 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     const uint16_t *s_src[2];
 #pragma unroll
     for (int ni = 0; ni < 2; ++ni) {
-        const int nt = nt_base + 2 * ni + (l32 >> 4);
+        // SWIGLU: every 16-column tile holds 8 gate columns, then the 8 matching up columns; sub-tile 0
+        // gathers the gate columns of the wavefront's four tiles, sub-tile 1 their up columns, so a lane
+        // holds a gate value and its up value in the same register of the two accumulators
+        const int nt = SWIGLU ? nt_base + (l32 >> 3) : nt_base + 2 * ni + (l32 >> 4);
+        const int c = SWIGLU ? (l32 & 7) + 8 * ni : (l32 & 15);
 #pragma unroll
-        for (int v = 0; v < 2; ++v) b_src[ni][v] = B + (size_t)nt * G * 64 + (l32 & 15) + 16 * (2 * v + h);
-        s_src[ni] = S + (size_t)nt * Gs * kTileN + (l32 & 15);
+        for (int v = 0; v < 2; ++v) b_src[ni][v] = B + (size_t)nt * G * 64 + c + 16 * (2 * v + h);
+        s_src[ni] = S + (size_t)nt * Gs * kTileN + c;
     }
     const int gs_mask = (Gs == 1) ? 0 : -1;
     // a zero scale would break the running rescale below; it is replaced by a

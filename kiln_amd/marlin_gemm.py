@@ -200,8 +200,8 @@ def unpack_to_gptq(b_packed, scales_tiled, groupsize: int = 128):
 
 def interleave_gate_up(gate_b, gate_s, up_b, up_s, groupsize: int = 128):
     """Two packed projections of equal shape `[k, n_each]` (gate, up) -> the packed `[k, 2 n_each]`
-    form `marlin_w4a16_gemm_swiglu` reads: per 64 columns, 32 gate columns then the 32 matching
-    up columns."""
+    form `marlin_w4a16_gemm_swiglu` reads: per 16 columns (one column tile), 8 gate columns then
+    the 8 matching up columns."""
     gate_b = np.ascontiguousarray(gate_b).view(np.int32)
     up_b = np.ascontiguousarray(up_b).view(np.int32)
     gate_s = np.ascontiguousarray(gate_s).view(np.float16)

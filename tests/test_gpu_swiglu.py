@@ -30,7 +30,9 @@ def _problem(oracle, m, k, n_out, g, seed, sigma=1.0):
 
 @pytest.mark.parametrize("m,k,n_out,g,sigma", [
     (1, 2560, 1024, 128, 1.0), (16, 2560, 1024, 128, 1.0), (32, 256, 256, -1, 1.0),
-    (33, 2560, 1024, 128, 1.0), (64, 2560, 9216, 128, 1.0), (100, 512, 256, 128, 1.0),
+    (4, 9216, 1280, 128, 1.0),      # K slices: the product is formed by the block that sums them
+    (16, 2560, 9216, 128, 1.0), (24, 2560, 9216, 128, 1.0), (40, 9216, 1280, 128, 1.0),
+    (33, 2560, 1024, 128, 1.0), (64, 2560, 9216, 128, 1.0), (100, 512, 256, 128, 1.0), (128, 2560, 9216, 128, 1.0),
     (300, 2560, 2560, 128, 0.5), (1000, 1024, 4096, 128, 0.5), (2048, 2560, 9216, 128, 0.5),
 ])
 def test_swiglu_cases(oracle, m, k, n_out, g, sigma):
@@ -55,7 +57,7 @@ def test_swiglu_matches_unfused_calls_and_repeats(oracle):
         h = marlin_gemm.marlin_w4a16_gemm_swiglu(xt, bt, st, g)
         for _ in range(3):
             assert torch.equal(marlin_gemm.marlin_w4a16_gemm_swiglu(xt, bt, st, g), h)
-        y = marlin_gemm.marlin_w4a16_gemm(xt, bt, st, g).float().reshape(m, n_out // 32, 2, 32)
+        y = marlin_gemm.marlin_w4a16_gemm(xt, bt, st, g).float().reshape(m, n_out // 8, 2, 8)
         unfused = (torch.nn.functional.silu(y[:, :, 0]) * y[:, :, 1]).reshape(m, n_out)
         scale = unfused.abs().amax(dim=1, keepdim=True)
         assert torch.all((h.float() - unfused).abs() <= 1e-2 * scale)

@@ -285,7 +285,7 @@ def test_repack_cli_converts_a_safetensors_shard(tmp_path, oracle):
 
 
 def test_interleave_gate_up_is_a_column_permutation(oracle):
-    """Dequantising the interleaved pack gives, per 64 columns, 32 gate columns then the 32
+    """Dequantising the interleaved pack gives, per 16 columns, 8 gate columns then the 8
     matching up columns; shapes outside n_each % 128 == 0 are rejected."""
     k, n_each, g = 256, 256, 128
     packs = []
@@ -299,9 +299,9 @@ def test_interleave_gate_up_is_a_column_permutation(oracle):
     q_gu, s_plain = pack.unpack_to_gptq(b_gu, s_gu, g)
     deq = oracle.c_dequant_f32(q_gu.view(np.uint32), np.asarray(s_plain).view(np.uint16), g)
     want = np.empty((k, 2 * n_each), np.float32)
-    for j in range(n_each // 32):
-        want[:, 64 * j:64 * j + 32] = packs[0][2][:, 32 * j:32 * j + 32]
-        want[:, 64 * j + 32:64 * j + 64] = packs[1][2][:, 32 * j:32 * j + 32]
+    for j in range(n_each // 8):
+        want[:, 16 * j:16 * j + 8] = packs[0][2][:, 8 * j:8 * j + 8]
+        want[:, 16 * j + 8:16 * j + 16] = packs[1][2][:, 8 * j:8 * j + 8]
     assert np.array_equal(deq, want)
     with pytest.raises(marlin_gemm.MarlinGemmError, match="shape"):
         pack.interleave_gate_up(packs[0][0][:, :2 * 192].copy(), packs[0][1][:, :192].copy(),
