@@ -67,7 +67,7 @@ TUNING_EXPORTS = (
     "kiln_w4a16_debug_prefill_min_m", "kiln_w4a16_debug_prefill_ks", "kiln_w4a16_debug_prefill_bn",
     "kiln_w4a16_debug_prefill_bm", "kiln_w4a16_debug_prefill_nb_full", "kiln_w4a16_debug_decode_direct_max_m",
     "kiln_w4a16_debug_decode_group_major", "kiln_w4a16_debug_decode_runs_per_launch", "kiln_w4a16_debug_tune",
-    "kiln_w4a16_debug_mid",
+    "kiln_w4a16_debug_mid", "kiln_w4a16_debug_gmp",
 )
 
 _libs: dict[bool, ctypes.CDLL] = {}
@@ -106,6 +106,7 @@ def use_shipped() -> None:
         L.kiln_w4a16_debug_decode_group_major(-1)
         L.kiln_w4a16_debug_decode_runs_per_launch(0)
         L.kiln_w4a16_debug_mid(-1, 0, 0)
+        L.kiln_w4a16_debug_gmp(0, 0, 0)
     _active_tuning = False
 
 
@@ -122,7 +123,7 @@ def _load(tuning: bool) -> ctypes.CDLL:
         for name in TUNING_EXPORTS:
             fn = getattr(L, name)
             fn.restype = None
-            fn.argtypes = [ctypes.c_int] * (3 if name in ("kiln_w4a16_debug_tune", "kiln_w4a16_debug_mid") else 1)
+            fn.argtypes = [ctypes.c_int] * (3 if name in ("kiln_w4a16_debug_tune", "kiln_w4a16_debug_mid", "kiln_w4a16_debug_gmp") else 1)
 
     c = ctypes
     vp, i = c.c_void_p, c.c_int

@@ -27,6 +27,7 @@ struct DecodeArgs {
     bool direct = false;  // operand fragments straight from L2 instead of an LDS-staged slice (few rows)
     bool regs = false;    // the plan is for the register-fragment group-major instance (M <= 32)
     int gm_tiles = 0;     // > 0: the plan is for the LDS-staged group-major instance, this many tiles per block
+    bool gmp = false;     // with gm_tiles > 0: the plan is for the private-staging group-major instance instead
     // optional low-rank term (r_total == 0: none): C += lora_t * lora_b^T
     const void *lora_t = nullptr;  // bf16 [lora_slices][lora_rows][r_total rounded up to 16], at this slab's first
                                    // row: scaled projection in K slices, padding columns zero
@@ -64,6 +65,8 @@ size_t decode_gmr_lds_bytes(int waves, int tiles, int slabs);
 bool decode_group_major_regs_ok(const struct DecodeArgs &a);  // ... and the one that takes up to 32 rows?
 int decode_max_tiles_per_block();
 hipError_t launch_decode(const DecodeArgs &args, hipStream_t stream);
+bool decode_gmp_ok(const DecodeArgs &a);                        // does the plan fit the private-staging instance?
+hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream);
 
 // One launch of the mid-M kernel: runs of up to 64 rows (grid z) against the whole weight.
 struct MidArgs {

@@ -43,6 +43,7 @@ struct DecodePlan {
     bool regs = false;  // for the register-fragment group-major instance
     long cost = -1;
     int gm_tiles = 0;   // > 0: for the LDS-staged group-major instance, tiles per block
+    bool gmp = false;   // with gm_tiles > 0: for the private-staging group-major instance
 };
 
 enum class DecodeMode { kStaged, kDirect, kRegs };
@@ -61,6 +62,7 @@ struct Tuning {
     int decode_runs_per_launch = 0;   // 1 = one run of rows per launch
     int prefill_ks = 0, prefill_bn = 0, prefill_bm = 0, prefill_nb_full = -1;
     int force_ks = 0, force_u = 0, force_waves = 0;
+    int gmp_tiles = 0, gmp_waves = 0, gmp_ks = 0;   // > 0: the private-staging small-M instance with this plan
     int mid = -1;                     // 0 = never the mid-M kernel, 1 = wherever a plan fits (any row count), -1 = automatic
     int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
 };
@@ -204,8 +206,72 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
 // handicapped by what the staged group-major instance measured faster on plans both can run.
 // 17 <= m <= 32: only the register-fragment instance takes that many rows; false if no plan fits.
 constexpr long kRegsHandicap = 8;
-bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, DecodePlan *plan, bool *direct) {
+// the private-staging group-major instance with a given plan, if the shape takes it
+bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, DecodePlan *plan) {
+    const int G = k / kGroupK, NT = n / kTileN;
+    if (ks < 1 || G % ks != 0 || tiles < 1) return false;
+    DecodeArgs a;
+    a.M = m;
+    a.N = n;
+    a.K = k;
+    a.KS = ks;
+    a.GS = G / ks;
+    a.waves = waves < a.GS ? waves : a.GS;
+    a.gm_tiles = tiles;
+    if (!decode_gmp_ok(a)) return false;
+    *plan = DecodePlan{};
+    plan->KS = ks;
+    plan->GS = a.GS;
+    plan->waves = a.waves;
+    plan->gm_tiles = tiles;
+    plan->U = tiles * ceil_div(a.GS, a.waves);
+    plan->BPS = ceil_div(NT, tiles);
+    plan->gmp = true;
+    return true;
+}
+
+// Best plan for the private-staging group-major instance (m <= 16).  Cost in microseconds, fitted
+// to a sweep of the model's projection shapes at 1, 4 and 16 rows: a launch costs about 2.8 us
+// beside its rounds of blocks; a block streams its T * GS KiB of weights at 0.036 us per KiB and
+// stages its rows of A from L2 (GS KiB per four rows) at 0.0125 us per KiB -- with 16 rows an
+// unsliced down projection stages four times the bytes it streams, which is why it is sliced there
+// and not at 4 rows; an exchange between K slices costs 2 us at two slices and 0.4 us more per
+// further slice (only two and three slices were measured).
+bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
+    const int G = k / kGroupK, NT = n / kTileN;
+    const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
+    static const int kWaves[] = {12, 16, 8};
+    float best_cost = -1.f;
+    for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
+        if (G % ks != 0) continue;
+        const int GS = G / ks;
+        for (int waves : kWaves) {
+            for (int T = 1; T <= 6; ++T) {
+                DecodePlan p;
+                if (!gmp_plan(m, n, k, T, waves, ks, &p)) continue;
+                const int rounds = ceil_div(ceil_div(NT, T) * ks, cus);
+                const float cost = 2.8f + rounds * (0.036f * T * GS + 0.0125f * a_kib_per_group * GS) +
+                                   (ks > 1 ? 1.2f + 0.4f * ks : 0.f);
+                if (best_cost < 0.f || cost < best_cost - 1e-4f) {
+                    best_cost = cost;
+                    *best = p;
+                }
+            }
+        }
+    }
+    return best_cost >= 0.f;
+}
+
+bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, bool lora, DecodePlan *plan,
+                   bool *direct) {
     *direct = false;
+    if (g_tune.gmp_tiles > 0 && m <= 16 && gmp_plan(m, n, k, g_tune.gmp_tiles, g_tune.gmp_waves, g_tune.gmp_ks, plan))
+        return true;
+    // up to 16 rows of a call without adapters or overrides: the private-staging instance
+    if (m <= 16 && !lora && thread_k <= 0 && thread_n <= 0 && g_tune.gmp_tiles == 0 && g_tune.decode_group_major == -1 &&
+        g_tune.decode_direct_max_m < 0 && !g_tune.force_ks && !g_tune.force_u && !g_tune.force_waves &&
+        plan_decode_gmp(m, n, k, cus, plan))
+        return true;
     const bool regs_allowed = g_tune.decode_group_major != 0 && g_tune.decode_group_major != 1 && thread_n <= 0;
     if (m > 16) return regs_allowed && plan_decode(n, k, cus, thread_k, thread_n, DecodeMode::kRegs, m, plan);
     if (g_tune.decode_direct_max_m >= 0 && m <= g_tune.decode_direct_max_m) {  // tuning override
@@ -232,15 +298,16 @@ bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, Dec
 // of host time each, more than the GEMM they plan, so they are kept: a small table behind a
 // mutex (the entry points may be entered from several threads at once).
 struct SlabKey {
-    int m, n, k, cus, thread_k, thread_n;
+    int m, n, k, cus, thread_k, thread_n, lora;
     bool operator==(const SlabKey &o) const {
-        return m == o.m && n == o.n && k == o.k && cus == o.cus && thread_k == o.thread_k && thread_n == o.thread_n;
+        return m == o.m && n == o.n && k == o.k && cus == o.cus && thread_k == o.thread_k && thread_n == o.thread_n &&
+               lora == o.lora;
     }
 };
 struct SlabKeyHash {
     size_t operator()(const SlabKey &key) const {
         size_t h = 1469598103934665603ull;
-        for (int v : {key.m, key.n, key.k, key.cus, key.thread_k, key.thread_n}) h = (h ^ (size_t)(unsigned)v) * 1099511628211ull;
+        for (int v : {key.m, key.n, key.k, key.cus, key.thread_k, key.thread_n, key.lora}) h = (h ^ (size_t)(unsigned)v) * 1099511628211ull;
         return h;
     }
 };
@@ -252,15 +319,15 @@ struct SlabChoice {
 std::mutex g_plan_mutex;
 std::unordered_map<SlabKey, SlabChoice, SlabKeyHash> g_plan_cache;
 
-SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n) {
-    const SlabKey key{m, n, k, cus, thread_k, thread_n};
+SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n, bool lora) {
+    const SlabKey key{m, n, k, cus, thread_k, thread_n, lora ? 1 : 0};
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         auto it = g_plan_cache.find(key);
         if (it != g_plan_cache.end()) return it->second;
     }
     SlabChoice c;
-    c.ok = choose_decode(m, n, k, cus, thread_k, thread_n, &c.plan, &c.direct);
+    c.ok = choose_decode(m, n, k, cus, thread_k, thread_n, lora, &c.plan, &c.direct);
     std::lock_guard<std::mutex> lock(g_plan_mutex);
     if (g_plan_cache.size() > 4096) g_plan_cache.clear();  // a caller cycling through many shapes
     g_plan_cache.emplace(key, c);
@@ -277,7 +344,7 @@ SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n)
 // runs (20.2...21.0).  Without such a plan the matrix-core kernel starts at 49 rows.
 bool takes_prefill(int m, int n, int k, int cus) {
     if (g_tune.prefill_min_m > 0) return m >= g_tune.prefill_min_m;
-    if (!slab_choice(32, n, k, cus, -1, -1).ok) return m >= 49;
+    if (!slab_choice(32, n, k, cus, -1, -1, false).ok) return m >= 49;
     if ((long)n * k > (32L << 20) && m >= 49 && m <= 64) return true;
     return m >= 81;
 }
@@ -429,10 +496,10 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, bool lo
         l.r0 = r0;
         l.M = left < 32 ? left : 32;
         SlabChoice c;
-        if (l.M > 16) c = slab_choice(l.M, n, k, cus, thread_k, thread_n);
+        if (l.M > 16) c = slab_choice(l.M, n, k, cus, thread_k, thread_n, lora);
         if (!c.ok) {
             l.M = left < 16 ? left : 16;
-            c = slab_choice(l.M, n, k, cus, thread_k, thread_n);
+            c = slab_choice(l.M, n, k, cus, thread_k, thread_n, lora);
             // no small-M plan (K beyond eight slices of 32 groups): the matrix-core kernel takes any M
             if (!c.ok) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
         }
@@ -649,8 +716,9 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         a.waves = l.plan.waves;
         a.regs = l.plan.regs;
         a.gm_tiles = l.plan.gm_tiles;
+        a.gmp = l.plan.gmp;
         a.group_major = g_tune.decode_group_major;
-        if (launch_decode(a, st) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
+        if ((a.gmp ? launch_decode_gmp(a, st) : launch_decode(a, st)) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
     }
     return KILN_W4A16_OK;
 }
@@ -746,13 +814,13 @@ kiln_marlin_status_t kiln_marlin_w4a16_gemm(const void *A, const void *B, void *
 // m <= 32; returns 0, or 1 if no plan fits.
 int kiln_w4a16_debug_decode_plan(int m, int n, int k, int cus, int *out) {
     if (m < 1 || m > 32 || cus < 1 || !shape_ok(n, k, 128)) return 1;
-    const SlabChoice c = slab_choice(m, n, k, cus, -1, -1);
+    const SlabChoice c = slab_choice(m, n, k, cus, -1, -1, false);
     if (!c.ok) return 1;
     const DecodePlan &p = c.plan;
     out[0] = p.KS; out[1] = p.GS; out[2] = p.U; out[3] = p.BPS; out[4] = p.waves;
     out[5] = c.direct;
     out[6] = p.regs;
-    out[7] = p.gm_tiles;
+    out[7] = p.gmp ? -p.gm_tiles : p.gm_tiles;   // negative: the private-staging instance
     return 0;
 }
 
@@ -786,6 +854,12 @@ void kiln_w4a16_debug_prefill_nb_full(int nb) { g_tune.prefill_nb_full = nb; }
 void kiln_w4a16_debug_decode_direct_max_m(int m) { g_tune.decode_direct_max_m = m; tuning_changed(); }
 void kiln_w4a16_debug_decode_group_major(int mode) { g_tune.decode_group_major = mode; tuning_changed(); }
 void kiln_w4a16_debug_decode_runs_per_launch(int runs) { g_tune.decode_runs_per_launch = runs; }
+void kiln_w4a16_debug_gmp(int tiles, int waves, int kslices) {
+    g_tune.gmp_tiles = tiles;
+    g_tune.gmp_waves = waves;
+    g_tune.gmp_ks = kslices;
+    tuning_changed();
+}
 void kiln_w4a16_debug_mid(int mode, int pairs, int kslices) {
     g_tune.mid = mode;
     g_tune.mid_pairs = pairs;

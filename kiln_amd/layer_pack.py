@@ -1,0 +1,157 @@
+"""Host mirror of the reference's load-time wiring of packed projections, widened to every
+quantisable linear of a layer.
+
+The reference queues only `q_proj` and the three MLP projections for the post-loop batch pack
+(crates/kiln-model/src/forward.rs:1884-1890, :2002-2018: `MarlinPackKind`, `MarlinPackEntry`),
+installs each packed weight into its `*_marlin` slot and drops the bf16 copy
+(`install_marlin_packed`, forward.rs:1736-1771), and leaves `k/v/o_proj` and the GDN
+projections on bf16 (forward.rs:1909-1980 builds them without a packed slot).  Here the same
+queue / batch pack / install sequence takes every projection of both layer kinds:
+
+    full attention   q_proj, k_proj, v_proj, o_proj
+    linear attention in_proj_qkv, in_proj_z, out_proj, in_proj_a, in_proj_b
+    MLP              gate_proj, up_proj, down_proj  (optionally gate and up as one fused,
+                     interleaved pack for the SwiGLU entry point)
+
+`shape_is_supported` (marlin_proj.rs:53-55) decides per projection: the 32-column
+`in_proj_a` / `in_proj_b` come back unpacked and stay on bf16, exactly the `None` the reference's
+`pack_from_bf16_batch` returns for an unsupported shape (marlin_proj.rs:229-262).  At run time
+`LayerProjections.forward` is what `mlp_proj_forward_decode_if` / `q_proj_forward_decode_if`
+(forward.rs:2923-2946, :4776-4801) are to the reference: packed GEMM where a packed weight is
+installed (with the LoRA delta fused when an adapter is attached), bf16 matmul otherwise.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from enum import Enum
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from . import marlin_gemm, marlin_proj
+from .lora import proj_forward
+from .marlin_proj import MarlinPackedProj, MarlinProjError
+
+
+class PackKind(Enum):
+    """`MarlinPackKind` (forward.rs:1720-1725) plus the projections the reference leaves on bf16."""
+    QProj = "q_proj"
+    KProj = "k_proj"
+    VProj = "v_proj"
+    OProj = "o_proj"
+    InProjQkv = "in_proj_qkv"
+    InProjZ = "in_proj_z"
+    OutProj = "out_proj"
+    InProjA = "in_proj_a"
+    InProjB = "in_proj_b"
+    GateProj = "gate_proj"
+    UpProj = "up_proj"
+    DownProj = "down_proj"
+
+
+FULL_ATTENTION_KINDS = (PackKind.QProj, PackKind.KProj, PackKind.VProj, PackKind.OProj)
+LINEAR_ATTENTION_KINDS = (PackKind.InProjQkv, PackKind.InProjZ, PackKind.OutProj, PackKind.InProjA, PackKind.InProjB)
+MLP_KINDS = (PackKind.GateProj, PackKind.UpProj, PackKind.DownProj)
+# what the reference itself queues (forward.rs:1884-1890, 2002-2018)
+REFERENCE_KINDS = (PackKind.QProj, PackKind.GateProj, PackKind.UpProj, PackKind.DownProj)
+
+
+@dataclass
+class PackEntry:
+    """`MarlinPackEntry` (forward.rs:1727-1731)."""
+    layer_idx: int
+    kind: PackKind
+
+
+@dataclass
+class LayerProjections:
+    """One layer's projections: `weights_t[kind]` is the pre-transposed `[k, n]` bf16 weight (the
+    reference's `*_proj_t`), `packed[kind]` the installed packed weight (its `*_proj_marlin`)."""
+    weights_t: Dict[PackKind, Optional[torch.Tensor]]
+    packed: Dict[PackKind, MarlinPackedProj] = field(default_factory=dict)
+    gate_up_fused: Optional[MarlinPackedProj] = None   # gate and up interleaved for the SwiGLU entry point
+
+    def is_packed(self, kind: PackKind) -> bool:
+        return kind in self.packed
+
+    def forward(self, kind: PackKind, x: torch.Tensor, lora=None, lora_scale: float = 1.0) -> torch.Tensor:
+        """Packed GEMM (LoRA delta fused) where a packed weight is installed, bf16 matmul otherwise
+        (forward.rs:2923-2946, :4776-4801)."""
+        w = self.packed.get(kind)
+        if w is not None:
+            return proj_forward(x, w, lora, lora_scale)
+        w_t = self.weights_t.get(kind)
+        if w_t is None:
+            raise MarlinProjError(f"layer_pack: {kind.value} has neither a packed nor a bf16 weight")
+        y = x @ w_t
+        if lora is not None:                                  # unfused, as the reference's bf16 branch
+            y = y + ((x @ lora.a.t().to(x.dtype)) @ lora.b.t().to(x.dtype)) * lora_scale
+        return y
+
+    def swiglu(self, x: torch.Tensor) -> torch.Tensor:
+        """`silu(gate_proj(x)) * up_proj(x)` (forward.rs:2771-2819): one fused launch on the
+        interleaved pack when it is installed, otherwise two projections and the elementwise ops."""
+        if self.gate_up_fused is not None:
+            w = self.gate_up_fused
+            x2 = x.reshape(-1, w.k).contiguous()
+            h = marlin_gemm.marlin_w4a16_gemm_swiglu(x2, w.b_packed, w.scales, w.groupsize)
+            return h.reshape(*x.shape[:-1], w.n // 2)
+        gate = self.forward(PackKind.GateProj, x)
+        up = self.forward(PackKind.UpProj, x)
+        return torch.nn.functional.silu(gate) * up
+
+
+def queue_layer(layer_idx: int, layer: LayerProjections, kinds: Optional[Sequence[PackKind]] = None,
+                groupsize: int = 128) -> Tuple[List[Tuple[torch.Tensor, int]], List[PackEntry]]:
+    """The per-layer part of the reference's build loop (forward.rs:1884-1890, 2002-2018): one pack
+    input and one sidecar entry per projection the layer has.  `kinds` = None queues every
+    projection; `REFERENCE_KINDS` reproduces the reference's own selection."""
+    inputs, meta = [], []
+    for kind, w_t in layer.weights_t.items():
+        if w_t is None or (kinds is not None and kind not in kinds):
+            continue
+        inputs.append((w_t, groupsize))
+        meta.append(PackEntry(layer_idx, kind))
+    return inputs, meta
+
+
+def install_packed(layer: LayerProjections, kind: PackKind, packed: MarlinPackedProj, drop_bf16: bool = True) -> None:
+    """`install_marlin_packed` (forward.rs:1736-1771): the packed weight goes into its slot and the
+    bf16 copy is dropped unless `drop_bf16` is off (`KILN_DISABLE_MARLIN_BF16_DROP`)."""
+    layer.packed[kind] = packed
+    if drop_bf16:
+        layer.weights_t[kind] = None
+
+
+def pack_layers(layers: Sequence[LayerProjections], kinds: Optional[Sequence[PackKind]] = None,
+                groupsize: int = 128, drop_bf16: bool = True, fuse_gate_up: bool = False) -> Dict[str, int]:
+    """The post-loop batch pack and install (forward.rs:2040-2085): every queued projection goes
+    through `pack_from_bf16_batch` (serial copies, threaded host pack); a projection whose shape the
+    kernels do not take (`shape_is_supported`, e.g. the 32-column `in_proj_a` / `in_proj_b`) comes
+    back as None and keeps its bf16 weight.  With `fuse_gate_up`, gate and up of a layer are also
+    interleaved into one pack for the SwiGLU entry point.  Returns counts for the caller's log line."""
+    inputs: List[Tuple[torch.Tensor, int]] = []
+    meta: List[PackEntry] = []
+    for i, layer in enumerate(layers):
+        li, lm = queue_layer(i, layer, kinds, groupsize)
+        inputs += li
+        meta += lm
+    packed = marlin_proj.pack_from_bf16_batch(inputs)
+    n_packed = 0
+    for entry, p in zip(meta, packed):
+        if p is not None:
+            install_packed(layers[entry.layer_idx], entry.kind, p, drop_bf16)
+            n_packed += 1
+    n_fused = 0
+    if fuse_gate_up:
+        for layer in layers:
+            g, u = layer.packed.get(PackKind.GateProj), layer.packed.get(PackKind.UpProj)
+            if g is None or u is None or g.k != u.k or g.n != u.n or g.n % 128 != 0:
+                continue
+            b_gu, s_gu = marlin_gemm.interleave_gate_up(g.b_packed.cpu().numpy(), g.scales.cpu().numpy(),
+                                                        u.b_packed.cpu().numpy(), u.scales.cpu().numpy(), g.groupsize)
+            dev = g.b_packed.device
+            layer.gate_up_fused = MarlinPackedProj(torch.from_numpy(b_gu).to(dev), torch.from_numpy(s_gu).to(dev),
+                                                   g.groupsize, g.k, 2 * g.n)
+            n_fused += 1
+    return {"inputs": len(inputs), "packed": n_packed, "kept_bf16": len(inputs) - n_packed, "gate_up_fused": n_fused}

@@ -1,0 +1,100 @@
+"""The load-time wiring of packed projections for both layer kinds (host mirror of
+crates/kiln-model/src/forward.rs:1884-2085 widened to k/v/o_proj and the GDN projections), on
+the model's real projection shapes, against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from kiln_amd import layer_pack
+from kiln_amd.layer_pack import LayerProjections, PackKind
+from tests.gpu_util import bf16_bits, bf16_tensor, row_errors
+
+pytestmark = pytest.mark.gpu
+
+HIDDEN = 2560
+# (k, n) of every projection: crates/kiln-core/src/config.rs:80-97 (16 heads x 256 gated -> 8192,
+# 4 kv heads x 256 = 1024, 32 value heads x 128 = 4096, 16 + 16 + 32 heads x 128 = 8192 for qkv)
+FULL = {PackKind.QProj: (HIDDEN, 8192), PackKind.KProj: (HIDDEN, 1024), PackKind.VProj: (HIDDEN, 1024),
+        PackKind.OProj: (4096, HIDDEN)}
+LINEAR = {PackKind.InProjQkv: (HIDDEN, 8192), PackKind.InProjZ: (HIDDEN, 4096), PackKind.OutProj: (4096, HIDDEN),
+          PackKind.InProjA: (HIDDEN, 32), PackKind.InProjB: (HIDDEN, 32)}
+MLP = {PackKind.GateProj: (HIDDEN, 9216), PackKind.UpProj: (HIDDEN, 9216), PackKind.DownProj: (9216, HIDDEN)}
+
+
+def _weights(oracle, shapes, seed):
+    host, dev = {}, {}
+    for i, (kind, (k, n)) in enumerate(shapes.items()):
+        w = oracle.c_lcg_fill(k * n, 0xC0FFEE5EED ^ (seed * 131 + i), 0.5).reshape(k, n)
+        bits = oracle.np_f32_to_bf16(w)
+        host[kind] = oracle.np_bf16_to_f32(bits)          # what the packer quantises: the bf16 weight
+        dev[kind] = bf16_tensor(bits)
+    return host, dev
+
+
+@pytest.fixture(scope="module")
+def packed_layers(oracle):
+    h0, d0 = _weights(oracle, {**FULL, **MLP}, 1)
+    h1, d1 = _weights(oracle, {**LINEAR, **MLP}, 2)
+    layers = [LayerProjections(d0), LayerProjections(d1)]
+    stats = layer_pack.pack_layers(layers, fuse_gate_up=True)
+    return layers, [h0, h1], stats
+
+
+def test_every_supported_projection_is_packed_and_the_rest_stay_bf16(packed_layers):
+    layers, _, stats = packed_layers
+    assert stats == {"inputs": 15, "packed": 13, "kept_bf16": 2, "gate_up_fused": 2}
+    full, linear = layers
+    for kind in (*FULL, *MLP):
+        assert full.is_packed(kind) and full.weights_t[kind] is None, kind        # bf16 copy dropped
+    for kind in (PackKind.InProjQkv, PackKind.InProjZ, PackKind.OutProj, *MLP):
+        assert linear.is_packed(kind), kind
+    for kind in (PackKind.InProjA, PackKind.InProjB):                             # n = 32: marlin_proj.rs:53-55
+        assert not linear.is_packed(kind) and linear.weights_t[kind] is not None
+    assert tuple(full.packed[PackKind.KProj].b_packed.shape) == (HIDDEN // 16, 2 * 1024)
+    assert tuple(full.packed[PackKind.KProj].scales.shape) == (HIDDEN // 128, 1024)
+
+
+def _check(oracle, layer, host_w, kind, m, seed):
+    k, n = host_w[kind].shape
+    x = oracle.gen_normal_bf16(m, k, 1.0, seed)
+    y = layer.forward(kind, bf16_tensor(x))
+    torch.cuda.synchronize()
+    assert tuple(y.shape) == (m, n)
+    if layer.is_packed(kind):
+        codes, s_bits, _ = oracle.c_quantize(host_w[kind], 128)
+        y_ref = oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128)
+    else:
+        y_ref = oracle.c_gemm_f32(x, host_w[kind])
+    err, yv, _ = row_errors(bf16_bits(y), y_ref, oracle)
+    assert np.all(np.isfinite(yv)) and err.max() <= 1e-2, (kind, m, err.max())
+
+
+@pytest.mark.parametrize("m", [1, 16, 512])
+@pytest.mark.parametrize("kind", [PackKind.KProj, PackKind.VProj])
+def test_kv_projections_n1024(oracle, packed_layers, kind, m):
+    layers, host, _ = packed_layers
+    _check(oracle, layers[0], host[0], kind, m, seed=m + 7)
+
+
+@pytest.mark.parametrize("layer_idx,kind", [(0, PackKind.QProj), (0, PackKind.OProj), (1, PackKind.InProjQkv),
+                                            (1, PackKind.InProjZ), (1, PackKind.OutProj), (1, PackKind.InProjA),
+                                            (1, PackKind.InProjB), (0, PackKind.DownProj)])
+def test_remaining_projections(oracle, packed_layers, layer_idx, kind):
+    layers, host, _ = packed_layers
+    for m in (1, 16):
+        _check(oracle, layers[layer_idx], host[layer_idx], kind, m, seed=m + layer_idx)
+    x3 = bf16_tensor(oracle.gen_normal_bf16(6, host[layer_idx][kind].shape[0], 1.0, 3)).reshape(2, 3, -1)
+    assert tuple(layers[layer_idx].forward(kind, x3).shape) == (2, 3, host[layer_idx][kind].shape[1])   # rank 3
+
+
+def test_fused_gate_up_swiglu_of_a_layer(oracle, packed_layers):
+    layers, host, _ = packed_layers
+    m = 16
+    x = oracle.gen_normal_bf16(m, HIDDEN, 1.0, 11)
+    h = layers[1].swiglu(bf16_tensor(x))
+    sides = []
+    for kind in (PackKind.GateProj, PackKind.UpProj):
+        codes, s_bits, _ = oracle.c_quantize(host[1][kind], 128)
+        sides.append(oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128))
+    err, _, _ = row_errors(bf16_bits(h), oracle.c_swiglu_f32(sides[0], sides[1]), oracle)
+    assert tuple(h.shape) == (m, 9216) and err.max() <= 1e-2

@@ -345,6 +345,15 @@ def test_decode_plans_are_launchable_and_keep_model_shapes_exchange_free():
                 assert rc == 0, (m, k, n, cus)
                 ks, gs, u, bps, waves, direct, regs, gm_tiles = list(out)
                 g, nt = k // 128, n // 16
+                if gm_tiles < 0:
+                    # the private-staging instance (m <= 16): whole tiles, equal slices of any length,
+                    # every wavefront one to six groups (three from three tiles on), at most 16 chunks
+                    tiles, gpw = -gm_tiles, -(-gs // waves)
+                    assert m <= 16 and not direct and not regs and ks * gs == g and 1 <= tiles <= 6
+                    assert 1 <= waves <= 16 and waves <= gs and gpw <= (6 if tiles <= 2 else 3) and tiles * gpw <= 16
+                    assert u == tiles * gpw and bps == -(-nt // tiles)
+                    assert waves * max(min(gpw, 3) * 4096, tiles * 1024) <= 159 * 1024
+                    continue
                 gs_last = g - (ks - 1) * gs
                 assert 1 <= ks <= 8 and 1 <= gs_last <= gs and (ks - 1) * gs < g
                 assert 1 <= u <= min(12, gs_last) and 1 <= waves <= 16
@@ -373,6 +382,9 @@ def test_decode_plans_are_launchable_and_keep_model_shapes_exchange_free():
         assert plan(m, 2560, 9216, 256, out) == 0
         ks, gs, u, bps, waves, _, regs, gm_tiles = list(out)
         assert ks * gs == 72 and (gm_tiles or (waves * u) % gs == 0) and ks * bps <= 256 and regs == (m > 16), list(out)
+    # few rows of the down projection run unsliced (nothing through the workspace); 16 rows are sliced
+    for m, want_ks in ((1, 1), (4, 1), (16, 3)):
+        assert plan(m, 2560, 9216, 256, out) == 0 and out[0] == want_ks and out[7] < 0, (m, list(out))
     assert plan(33, 2560, 2560, 256, out) == 1 and plan(16, 2560, 100, 256, out) == 1
 
 
@@ -419,12 +431,36 @@ def test_shipped_library_has_no_tuning_setters():
 
 
 def test_long_k_falls_back_to_the_matrix_core_path():
-    """K beyond eight slices of 32 groups has no small-M plan; such a GEMM takes the matrix-core
-    kernel at any row count instead of failing (the reference accepts any k % 128 == 0)."""
+    """A K that no small-M instance can slice has no small-M plan; such a GEMM takes the
+    matrix-core kernel at any row count instead of failing (the reference accepts any k % 128 == 0)."""
     L = _lib.load()
     out = (ctypes.c_int * 8)()
-    for k in (32896, 40960):
-        for m in (1, 16, 48):
-            assert L.kiln_w4a16_debug_gemm_plan(m, 2560, k, 256, out) == 0
-            assert out[0] == 1, (m, k, list(out))
+    for m in (1, 16, 48):               # 257 groups: no equal slicing fits any small-M instance
+        assert L.kiln_w4a16_debug_gemm_plan(m, 2560, 32896, 256, out) == 0
+        assert out[0] == 1, (m, list(out))
+    for m in (1, 16):                   # 320 groups = 8 slices of 40: the private-staging instance takes them
+        assert L.kiln_w4a16_debug_gemm_plan(m, 2560, 40960, 256, out) == 0
+        assert out[0] == 0 and out[1] == 1, (m, list(out))
     assert L.kiln_w4a16_debug_gemm_plan(16, 2560, 9216, 256, out) == 0 and out[0] == 0 and out[1] == 1
+
+
+def test_layer_wiring_keeps_bf16_without_a_gpu_and_reproduces_the_reference_selection():
+    """Host logic of the layer-level wiring (no GPU): weights that are not on the GPU come back
+    unpacked (marlin_proj.rs:91-93) and every projection stays on its bf16 matmul; the reference's
+    own selection queues q_proj and the three MLP projections only (forward.rs:1884-1890, 2002-2018)."""
+    import torch
+    from kiln_amd import layer_pack
+    from kiln_amd.layer_pack import LayerProjections, PackKind
+    torch.manual_seed(0)
+    shapes = {PackKind.QProj: (256, 512), PackKind.KProj: (256, 256), PackKind.InProjA: (256, 32),
+              PackKind.GateProj: (256, 512), PackKind.UpProj: (256, 512), PackKind.DownProj: (512, 256)}
+    layer = LayerProjections({kind: torch.randn(k, n).to(torch.bfloat16) for kind, (k, n) in shapes.items()})
+    inputs, meta = layer_pack.queue_layer(3, layer, layer_pack.REFERENCE_KINDS)
+    assert [e.kind for e in meta] == [PackKind.QProj, PackKind.GateProj, PackKind.UpProj, PackKind.DownProj]
+    assert all(e.layer_idx == 3 for e in meta) and all(g == 128 for _, g in inputs)
+    stats = layer_pack.pack_layers([layer])
+    assert stats == {"inputs": 6, "packed": 0, "kept_bf16": 6, "gate_up_fused": 0}
+    x = torch.randn(2, 3, 256).to(torch.bfloat16)
+    y = layer.forward(PackKind.KProj, x)
+    assert tuple(y.shape) == (2, 3, 256) and torch.equal(y, x @ layer.weights_t[PackKind.KProj])
+    assert marlin_proj.shape_is_supported(2560, 1024) and not marlin_proj.shape_is_supported(2560, 32)
