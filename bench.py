@@ -131,6 +131,23 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
     extra["m16_gate_up_eager_200_launches"] = {
         "event_us_p10": round(us[20], 2), "event_us_median": round(us[100], 2), "event_us_p90": round(us[180], 2),
         "wrapper_inclusive_wall_us": round(wall, 2)}
+    # host time of the C entry point alone (plan lookup + launch, no wrapper, no synchronisation):
+    # 2000 back-to-back calls on one stream, wall time per call
+    from kiln_amd import _lib
+    L = _lib.load()
+    st = torch.cuda.current_stream().cuda_stream
+    wsz = L.kiln_w4a16_workspace_bytes(16, 18432, 2560)
+    wbuf = torch.zeros(wsz, dtype=torch.uint8, device=dev)
+    b0, s0 = ws_[0]
+    for n_calls in (50, 2000):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_calls):
+            L.kiln_marlin_w4a16_gemm(x_.data_ptr(), b0.data_ptr(), o_.data_ptr(), s0.data_ptr(), 16, 18432, 2560,
+                                     wbuf.data_ptr(), GROUP, 0, st, -1, -1, -1, 16)
+        host = (time.perf_counter() - t0) / n_calls * 1e6
+        torch.cuda.synchronize()
+    extra["m16_gate_up_c_entry_host_us_per_call"] = round(host, 2)
     return extra
 
 
@@ -143,11 +160,13 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the legs reported under `extra` (every launch is then an M=16 launch of the workload)")
-    ap.add_argument("--profile", choices=["decode", "prefill", "lora"], default=None,
+    ap.add_argument("--profile", choices=["decode", "decode_m1", "mid", "prefill", "lora"], default=None,
                     help="for rocprofv3: launch K eager steps of the chosen regime (no graph, no CPU "
                          "baseline, no extra legs) plus one 64 MiB device copy that calibrates the "
-                         "memory-traffic counters, print no JSON; lora: the decode step and the M=512 "
-                         "gate+up GEMM, each with two stacked adapters (ranks 16 and 32)")
+                         "memory-traffic counters, print no JSON; decode_m1: gate+up, down and the "
+                         "2560x2560 GEMV at M=1; mid: the four projection shapes of the sweep at M=64; "
+                         "lora: the decode step and the M=512 gate+up GEMM, each with two stacked "
+                         "adapters (ranks 16 and 32)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build measures one GPU only (the path has no multi-GPU code); "
@@ -197,6 +216,25 @@ def main() -> int:
         if args.profile == "decode":
             for i in range(args.steps):
                 step(i)
+        elif args.profile == "decode_m1":
+            x1 = {name: torch.randn(1, kn[0], device=dev).to(torch.bfloat16) for name, kn in shapes.items()}
+            o1 = {name: torch.empty(1, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in shapes.items()}
+            sq = [make_layer(2560, 2560) for _ in range(LAYERS)]
+            xs, os_ = torch.randn(1, 2560, device=dev).to(torch.bfloat16), torch.empty(1, 2560, dtype=torch.bfloat16, device=dev)
+            for i in range(args.steps):
+                for name in shapes:
+                    b, s = layers[i % LAYERS][name]
+                    marlin_gemm.marlin_w4a16_gemm(x1[name], b, s, GROUP, out=o1[name])
+                marlin_gemm.marlin_w4a16_gemm(xs, sq[i % LAYERS][0], sq[i % LAYERS][1], GROUP, out=os_)
+        elif args.profile == "mid":
+            sweep = {"in_proj": (2560, 8192), "out_proj": (4096, 2560), **shapes}
+            sw = {name: [make_layer(*kn) for _ in range(8)] for name, kn in sweep.items() if name not in shapes}
+            x64 = {name: torch.randn(64, kn[0], device=dev).to(torch.bfloat16) for name, kn in sweep.items()}
+            o64 = {name: torch.empty(64, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in sweep.items()}
+            for i in range(args.steps):
+                for name in sweep:
+                    b, s = layers[i % LAYERS][name] if name in shapes else sw[name][i % 8]
+                    marlin_gemm.marlin_w4a16_gemm(x64[name], b, s, GROUP, out=o64[name])
         elif args.profile == "lora":
             ranks, lscales = (16, 32), (0.5, 1.0)
             ad = {name: ((torch.randn(sum(ranks), kn[0], device=dev) * 0.02).to(torch.bfloat16),
@@ -351,7 +389,7 @@ def main() -> int:
                    "wall_ms_per_step": round(wall_step / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_M16_TRAFFIC_BYTES,
-                     "kernel": "w4a16_decode_gm_kernel<5, 2, false> (gate+up, M=16, K=2560, N=18432)",
+                     "kernel": "w4a16_decode_gmp_kernel<5, 2, 4> (gate+up, M=16, K=2560, N=18432)",
                      "us_per_launch": round(us_gu, 3), "algorithmic_bytes_per_launch": bytes_gu},
         "cpu_baseline": cpu_baseline,
         "extra": extra,

@@ -235,8 +235,9 @@ bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, DecodePlan *pla
 // beside its rounds of blocks; a block streams its T * GS KiB of weights at 0.036 us per KiB and
 // stages its rows of A from L2 (GS KiB per four rows) at 0.0125 us per KiB -- with 16 rows an
 // unsliced down projection stages four times the bytes it streams, which is why it is sliced there
-// and not at 4 rows; an exchange between K slices costs 2 us at two slices and 0.4 us more per
-// further slice (only two and three slices were measured).
+// and not at 4 rows; a wavefront's chunks run one after the other (0.08 us each); an exchange
+// between K slices costs 2 us at two slices and 0.4 us more per further slice (the down projection
+// at 16 rows: 8.2 us in three slices, 9.2 in four, 9.9 in six, 11.2 in eight).
 bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
     const int G = k / kGroupK, NT = n / kTileN;
     const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
@@ -247,11 +248,14 @@ bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
         const int GS = G / ks;
         for (int waves : kWaves) {
             for (int T = 1; T <= 6; ++T) {
+                // 16 wavefronts only where they take one tile and the same number of groups each
+                // (out-projection: 4.9 against 5.3 us with 12); elsewhere they measured slower
+                if (waves == 16 && (T != 1 || GS % 16 != 0)) continue;
                 DecodePlan p;
                 if (!gmp_plan(m, n, k, T, waves, ks, &p)) continue;
                 const int rounds = ceil_div(ceil_div(NT, T) * ks, cus);
                 const float cost = 2.8f + rounds * (0.036f * T * GS + 0.0125f * a_kib_per_group * GS) +
-                                   (ks > 1 ? 1.2f + 0.4f * ks : 0.f);
+                                   0.08f * T * ceil_div(GS, p.waves) + (ks > 1 ? 1.2f + 0.4f * ks : 0.f);
                 if (best_cost < 0.f || cost < best_cost - 1e-4f) {
                     best_cost = cost;
                     *best = p;

@@ -26,19 +26,25 @@ namespace {
 
 constexpr int kGmpMaxWaves = 16;
 constexpr int kGmpSlotBytes = 16 * 256;  // one group of A: 16 rows x 128 bf16
-constexpr int kGmpHead = 3;              // chunks requested ahead of the one being consumed
+#ifndef KILN_GMP_HEAD
+#define KILN_GMP_HEAD 3
+#endif
+constexpr int kGmpHead = KILN_GMP_HEAD;  // chunks requested ahead of the one being consumed
 constexpr int kGmpMaxChunks = 16;        // chunks per wavefront, at most (straight-line code)
 
 // Issue order of a wavefront's loads (chunk j = group j / T, tile j % T: 2 loads each; A(g): AQ
-// LDS-direct loads; NS slots of A):
-//   before the first step: chunks 0 ... HEAD - 1, then A(0) ... A(NS - 1);
-//   step j: chunk j + HEAD; at the start of group g = j / T: [wait for A(g)], fragments to
-//   registers, A(g + NS) into the slot just read; then [wait for chunk j], products.
+// LDS-direct loads into slot g % 2):
+//   before the first step: chunks 0 ... HEAD - 1, then A(0);
+//   step j: chunk j + HEAD; at the start of group g = j / T: A(g + 1) (its slot's last reader,
+//   group g - 1, is done), [wait for A(g)], fragments to registers; then [wait for chunk j], products.
+// The activations of a group are requested one group ahead, not all at once: every block stages
+// its own copy of the slice, as many bytes through L2 as the weights at 16 rows, and a burst of
+// them at the start keeps the wavefronts in the issue stage while the weight stream runs dry.
 struct GmpSchedule {
     int wait_a[kGmpMaxChunks];      // by group
     int wait_chunk[kGmpMaxChunks];  // by chunk
 };
-constexpr GmpSchedule gmp_schedule(int T, int groups, int NS, int AQ) {
+constexpr GmpSchedule gmp_schedule(int T, int groups, int AQ) {
     const int U = T * groups;
     int kind[3 * kGmpMaxChunks] = {}, idx[3 * kGmpMaxChunks] = {}, size[3 * kGmpMaxChunks] = {};
     int n = 0;
@@ -58,25 +64,25 @@ constexpr GmpSchedule gmp_schedule(int T, int groups, int NS, int AQ) {
         return after;
     };
     for (int j = 0; j < kGmpHead && j < U; ++j) push(1, j, 2);
-    for (int g = 0; g < NS && g < groups; ++g) push(0, g, AQ);
+    push(0, 0, AQ);
     GmpSchedule s{};
     for (int j = 0; j < U; ++j) {
         if (j + kGmpHead < U) push(1, j + kGmpHead, 2);
         if (j % T == 0) {
             const int g = j / T;
+            if (g + 1 < groups) push(0, g + 1, AQ);
             s.wait_a[g] = issued_after(0, g);
-            if (g + NS < groups) push(0, g + NS, AQ);
         }
         s.wait_chunk[j] = issued_after(1, j);
     }
     return s;
 }
-template <int T, int GROUPS, int NS, int AQ>
+template <int T, int GROUPS, int AQ>
 struct GmpScheduleOf {
-    static constexpr GmpSchedule value = gmp_schedule(T, GROUPS, NS, AQ);
+    static constexpr GmpSchedule value = gmp_schedule(T, GROUPS, AQ);
 };
 
-constexpr int gmp_slots(int gpw) { return gpw < 3 ? gpw : 3; }
+constexpr int gmp_slots(int gpw) { return gpw < 2 ? gpw : 2; }
 
 // T tiles per block, GPW groups per wavefront (the first `full_waves` wavefronts; the others one
 // fewer), AQ = LDS-direct loads per group of A: 4 (16 rows), 2 (M <= 8) or 1 (M <= 4: rows 0...3
@@ -105,6 +111,7 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     // tile and never stored.  Four register sets rotate.
     u32x4 w[kGmpHead + 1];
     uint32_t sc[kGmpHead + 1];
+    static_assert(2 * kGmpHead + 8 <= 63, "outstanding loads must fit the wait counter");
     const uint32_t b_lane = lane * 16, s_lane = (lane & 15) * 2;
     auto request_chunk = [&](auto jc) {
         constexpr int j = decltype(jc)::value;
@@ -142,10 +149,9 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     // Straight-line code from the first request to the last use, one instance per group count.
     auto run = [&](auto nc) {
         constexpr int NGR = decltype(nc)::value, U = T * NGR;
-        using Sch = GmpScheduleOf<T, NGR, NS, AQ>;
+        using Sch = GmpScheduleOf<T, NGR, AQ>;
         unrolled<0, (kGmpHead < U ? kGmpHead : U)>(request_chunk);
-#pragma unroll
-        for (int g = 0; g < (NS < NGR ? NS : NGR); ++g) request_a(g, g);
+        request_a(0, 0);
         u32x4 af[4];
         f32x4 offset_term;
         unrolled<0, U>([&](auto jc) {
@@ -153,15 +159,12 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             constexpr int gi = j / T, ti = j % T, set = j % (kGmpHead + 1);
             if constexpr (j + kGmpHead < U) request_chunk(std::integral_constant<int, j + kGmpHead>{});
             if constexpr (ti == 0) {  // next group: fragments of its activations and its offset term
+                if constexpr (gi + 1 < NGR) request_a(gi + 1, (gi + 1) % NS);  // one group ahead
                 wait_vector_loads<Sch::value.wait_a[gi]>();
                 const unsigned char *ap = mine + (gi % NS) * kGmpSlotBytes + (lane & 15) * 256;
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
                     af[t] = *reinterpret_cast<const u32x4 *>(ap + (((4 * t + (lane >> 4)) ^ (lane & 15)) << 4));
-                if constexpr (gi + NS < NGR) {
-                    wait_lds_reads();  // the slot is free again
-                    request_a(gi + NS, gi % NS);
-                }
                 offset_term = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
