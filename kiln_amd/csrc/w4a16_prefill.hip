@@ -390,10 +390,13 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     // four stages form a ring and loads run three stages ahead of the products
     // (a stage lasts about as long as one L2 round trip, so a shallower
     // pipeline leaves the matrix cores waiting at every barrier).
-    // Unit c of row r is stored at unit position c ^ ((r >> 1) & 3); together
-    // with the two rows per 128-byte line this makes the 128-bit fragment reads
-    // bank-conflict free.  One direct load moves 1 KiB = 16 rows: lane i writes
-    // LDS slot i, so it fetches row i / 4, unit (i % 4) ^ ((i / 8) & 3).
+    // Unit c of row r is stored at unit position c ^ ((r >> 2) & 3): with four units
+    // per row, any 16 consecutive rows read at one unit index then touch the 16
+    // different 16-byte positions of a 256-byte bank line, so the 128-bit fragment
+    // reads are bank-conflict free (with (r >> 1) & 3 rows r and r + 8 collided: four
+    // conflict cycles on every fragment read, 13 % of the launch's cycles).  One direct
+    // load moves 1 KiB = 16 rows: lane i writes LDS slot i, so it fetches row i / 4,
+    // unit (i % 4) ^ ((i / 16) & 3).
     // Wavefront w moves the 16-row blocks w, w + NW, ...
     // Rows past M re-read row M - 1: their products are never stored.
     const uint16_t *a_src[APW];
@@ -402,7 +405,7 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
         const int blk = wave + NW * p;
         int row = m0 + blk * 16 + (lane >> 2);
         row = row < M ? row : M - 1;
-        a_src[p] = A + (size_t)row * K + (size_t)g_begin * kGroupK + (((lane & 3) ^ ((lane >> 3) & 3)) * 8);
+        a_src[p] = A + (size_t)row * K + (size_t)g_begin * kGroupK + (((lane & 3) ^ ((lane >> 4) & 3)) * 8);
     }
     const int n_stages = 4 * (g_end - g_begin);
     const unsigned lds_base = (unsigned)(size_t)(lds_ptr_t)lds;
@@ -438,11 +441,11 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
 
     const DequantConsts dq = dequant_consts();
     // fragment read offsets inside a stage for the two k16 steps of a stage:
-    // row (wm*MI*32 + mi*32 + l32), unit (2*step + h) ^ ((row >> 1) & 3)
+    // row (wm*MI*32 + mi*32 + l32), unit (2*step + h) ^ ((row >> 2) & 3)
     int a_off[2];
 #pragma unroll
     for (int sp = 0; sp < 2; ++sp)
-        a_off[sp] = (wm * MI * 32 + l32) * 64 + (((2 * sp + h) ^ ((l32 >> 1) & 3)) * 16);
+        a_off[sp] = (wm * MI * 32 + l32) * 64 + (((2 * sp + h) ^ ((l32 >> 2) & 3)) * 16);
 
     f32x16 acc[MI][2];
 #pragma unroll
@@ -503,7 +506,7 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
 #pragma unroll
                 for (int rr = 0; rr < RPW / 16; ++rr) {
                     const int row = wave * RPW + rr * 16 + (lane >> 2);
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(slot + row * 64 + (((lane & 3) ^ ((row >> 1) & 3)) * 16));
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(slot + row * 64 + (((lane & 3) ^ ((row >> 2) & 3)) * 16));
                     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
                     float s8 = 0.f;
 #pragma unroll
