@@ -49,7 +49,7 @@ typedef int kiln_marlin_status_t;
 #define KILN_W4A16_ERR_SCRATCH      6  /* the call needs more scratch than the library's static array holds */
 
 /* Size of the static device array behind kiln_marlin_w4a16_gemm_static_scratch (per GPU). */
-#define KILN_W4A16_STATIC_SCRATCH_BYTES (4u << 20)
+#define KILN_W4A16_STATIC_SCRATCH_BYTES (8u << 20)
 
 /*
  * C = A * dequant(B, s).

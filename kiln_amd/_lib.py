@@ -54,7 +54,7 @@ PROJ_EXPORTS = (
 
 PROJ_OK, PROJ_SKIPPED, PROJ_ERR = 0, 1, -1
 
-STATIC_SCRATCH_BYTES = 4 << 20   # KILN_W4A16_STATIC_SCRATCH_BYTES
+STATIC_SCRATCH_BYTES = 8 << 20   # KILN_W4A16_STATIC_SCRATCH_BYTES
 
 OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_LAUNCH, ERR_ARGUMENT, ERR_ZERO_POINT, ERR_SCRATCH = range(7)
 
@@ -67,7 +67,7 @@ TUNING_EXPORTS = (
     "kiln_w4a16_debug_prefill_min_m", "kiln_w4a16_debug_prefill_ks", "kiln_w4a16_debug_prefill_bn",
     "kiln_w4a16_debug_prefill_bm", "kiln_w4a16_debug_prefill_nb_full", "kiln_w4a16_debug_decode_direct_max_m",
     "kiln_w4a16_debug_decode_group_major", "kiln_w4a16_debug_decode_runs_per_launch", "kiln_w4a16_debug_tune",
-    "kiln_w4a16_debug_mid", "kiln_w4a16_debug_gmp",
+    "kiln_w4a16_debug_mid", "kiln_w4a16_debug_gmp", "kiln_w4a16_debug_flagged",
 )
 
 _libs: dict[bool, ctypes.CDLL] = {}
@@ -107,6 +107,7 @@ def use_shipped() -> None:
         L.kiln_w4a16_debug_decode_runs_per_launch(0)
         L.kiln_w4a16_debug_mid(-1, 0, 0)
         L.kiln_w4a16_debug_gmp(0, 0, 0)
+        L.kiln_w4a16_debug_flagged(-1)
     _active_tuning = False
 
 

@@ -8,6 +8,14 @@
 namespace kiln {
 
 // One launch of the decode kernel: M <= 16 rows of A against the whole weight.
+constexpr int kDecodeFlaggedMaxSlices = 4;
+
+// Counter-free exchange: blocks go to the eight dies round-robin by linear index (x fastest, then
+// the slice), and the slices of a tile should sit on different dies.  Slice ks takes column block
+// (x + ks * shift) % column_blocks; consecutive slices of a tile are then column_blocks - shift
+// block indices apart, which must be odd to differ modulo 8 for up to eight slices.
+inline int exchange_column_shift(int column_blocks) { return column_blocks % 2 == 0 ? 1 : 0; }
+
 struct DecodeArgs {
     const void *A;      // bf16 [M, K]
     const void *B;      // packed weights, tile layout
@@ -28,6 +36,8 @@ struct DecodeArgs {
     bool regs = false;    // the plan is for the register-fragment group-major instance (M <= 32)
     int gm_tiles = 0;     // > 0: the plan is for the LDS-staged group-major instance, this many tiles per block
     bool gmp = false;     // with gm_tiles > 0: the plan is for the private-staging group-major instance instead
+    bool flagged = false; // gmp with KS > 1: `partial` is all zero between launches and the parts are their own
+                          // arrival flags ((KS - 1) * N/16 * 1 KiB, KS <= kDecodeFlaggedMaxSlices); no counters
     // optional low-rank term (r_total == 0: none): C += lora_t * lora_b^T
     const void *lora_t = nullptr;  // bf16 [lora_slices][lora_rows][r_total rounded up to 16], at this slab's first
                                    // row: scaled projection in K slices, padding columns zero
@@ -82,7 +92,10 @@ struct MidArgs {
     int waves;          // wavefronts per block, <= 8 and <= GS; each owns ceil(GS / waves) groups or one fewer
     int pairs;          // pairs of 16-column tiles per block: 1, 2 or 3
     bool swiglu;        // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
+    bool flagged = false;  // KS > 1: `partial` is all zero between launches and the parts are their own arrival
+                           // flags ((KS - 1) slices of mid_partial_bytes() / KS each); needs mid_flagged_ok()
 };
+bool mid_flagged_ok(const MidArgs &a);
 int mid_column_blocks(const MidArgs &a);
 int mid_max_rows_per_run();
 bool mid_plan_ok(const MidArgs &a);

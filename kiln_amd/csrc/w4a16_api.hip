@@ -14,6 +14,11 @@ namespace {
 
 constexpr int kMaxDevices = 16;
 constexpr size_t kCounterBytes = 64 * 1024;   // arrival counters at the start of the workspace
+// Behind the counters: the region in which K slices exchange partial tiles without counters.  It is
+// all zero whenever no launch is running (the caller zero-fills it once with the counters; the
+// wavefront that adds a tile's parts writes zeros back), and a written word is never zero.
+constexpr size_t kFlaggedBytes = 4 * 1024 * 1024;
+constexpr size_t kZeroedBytes = kCounterBytes + kFlaggedBytes;
 
 struct DeviceInfo {
     std::once_flag once;
@@ -65,6 +70,7 @@ struct Tuning {
     int gmp_tiles = 0, gmp_waves = 0, gmp_ks = 0;   // > 0: the private-staging small-M instance with this plan
     int mid = -1;                     // 0 = never the mid-M kernel, 1 = wherever a plan fits (any row count), -1 = automatic
     int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
+    int flagged = -1;                 // 0 = K slices always meet through counters, -1 = automatic
 };
 #ifdef KILN_W4A16_TUNING_HOOKS
 Tuning g_tune;
@@ -230,14 +236,22 @@ bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, DecodePlan *pla
     return true;
 }
 
+// Can ks slices of n columns exchange their 16-row partial tiles in the zeroed region (every slice
+// but the last writes there)?
+bool flagged_exchange_fits(int ks, int n) {
+    return g_tune.flagged != 0 && ks > 1 && ks <= kDecodeFlaggedMaxSlices &&
+           (size_t)(ks - 1) * (n / kTileN) * 256 * sizeof(float) <= kFlaggedBytes;
+}
+
 // Best plan for the private-staging group-major instance (m <= 16).  Cost in microseconds, fitted
-// to a sweep of the model's projection shapes at 1, 4 and 16 rows: a launch costs about 2.8 us
+// to sweeps of the model's projection shapes at 1, 4, 8 and 16 rows: a launch costs about 2.8 us
 // beside its rounds of blocks; a block streams its T * GS KiB of weights at 0.036 us per KiB and
 // stages its rows of A from L2 (GS KiB per four rows) at 0.0125 us per KiB -- with 16 rows an
 // unsliced down projection stages four times the bytes it streams, which is why it is sliced there
-// and not at 4 rows; a wavefront's chunks run one after the other (0.08 us each); an exchange
-// between K slices costs 2 us at two slices and 0.4 us more per further slice (the down projection
-// at 16 rows: 8.2 us in three slices, 9.2 in four, 9.9 in six, 11.2 in eight).
+// and not at 4 rows; a wavefront's chunks run one after the other (0.08 us each); the exchange
+// between K slices is priced where the cost is formed (down projection at 16 rows in three
+// slices: 7.1 us with the parts as their own arrival flags, 8.4 through counters; four, six, eight
+// slices through counters 9.2, 9.9, 11.2).
 bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
     const int G = k / kGroupK, NT = n / kTileN;
     const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
@@ -254,8 +268,17 @@ bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
                 DecodePlan p;
                 if (!gmp_plan(m, n, k, T, waves, ks, &p)) continue;
                 const int rounds = ceil_div(ceil_div(NT, T) * ks, cus);
+                // The exchange: through counters 0.4 us per slice + 1.2; with the parts as their own
+                // arrival flags it grows with the tiles polled, 0.0037 us per (slice - 1) and tile
+                // (down projection, 160 tiles: 0.4 / 1.1 / 1.9 us at two / three / four slices;
+                // in-projection, 512 tiles: 2.0 us at two), + 0.3 because the unsliced estimates
+                // run high.  At up to four rows the additive model puts sliced plans 1 us too low
+                // (down projection: 6.7 us in three slices against 5.7 unsliced): + 0.7 there.
+                const bool flagged = flagged_exchange_fits(ks, n);
+                const float exchange = ks == 1 ? 0.f : (flagged ? 0.4f + 0.0037f * (ks - 1) * NT : 0.4f * ks + 1.2f) +
+                                                           (a_kib_per_group == 1 ? 0.7f : 0.f);
                 const float cost = 2.8f + rounds * (0.036f * T * GS + 0.0125f * a_kib_per_group * GS) +
-                                   0.08f * T * ceil_div(GS, p.waves) + (ks > 1 ? 1.2f + 0.4f * ks : 0.f);
+                                   0.08f * T * ceil_div(GS, p.waves) + exchange;
                 if (best_cost < 0.f || cost < best_cost - 1e-4f) {
                     best_cost = cost;
                     *best = p;
@@ -381,8 +404,12 @@ struct GemmPlan {
 
 // f32 partial tiles one small-M launch may exchange: per run and K slice two parts of N x 16.
 // Plans of whole tiles in one slice exchange nothing.
+// Do the K slices of this launch meet in the zeroed region, the parts being their own arrival flags?
+bool launch_flagged(const DecodeLaunch &l, int n) { return l.plan.gmp && flagged_exchange_fits(l.plan.KS, n); }
+
 size_t decode_launch_partial_bytes(const DecodeLaunch &l, int n, int k) {
     const DecodePlan &p = l.plan;
+    if (launch_flagged(l, n)) return 0;
     bool exchanges = p.KS > 1;
     if (!p.regs && p.gm_tiles == 0) {  // tile-major runs: blocks may cut tiles
         const int G = k / kGroupK, gs_last = G - (p.KS - 1) * p.GS, R = p.waves * p.U;
@@ -420,13 +447,19 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // projection does not (38.8 against 34.5).
 constexpr int kMidMinM = 33, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN = 8192;
 
+// Do the K slices of this mid-M launch meet in the zeroed region, the parts being their own arrival flags?
+bool mid_flagged(const MidArgs &a) {
+    return g_tune.flagged != 0 && mid_flagged_ok(a) && mid_partial_bytes(a) <= kFlaggedBytes;
+}
+
 // Plan for the mid-M kernel: pairs of tiles per block, K slices, wavefronts.  Cost in microseconds,
 // fitted to a sweep of the four projection shapes at 33...192 rows: a wavefront's group step is
 // bound by the round trip of its activations through L2 and by the products of its pairs
 // (0.75 + 0.55 us per pair; every block re-reads its rows of A, so fewer and wider blocks trade
 // parallelism for L2 traffic); a launch costs about 4.5 us beside its rounds of blocks, an exchange
-// between K slices 1.5 us at two slices and 1.7 us more per further slice (out-projection at 64
-// rows: 11.5 us unsliced, 10.4 in two slices, 13.8 in four).
+// between K slices through counters 1.5 us at two slices and 1.7 us more per further slice
+// (out-projection at 64 rows: 11.5 us unsliced, 10.4 in two slices, 13.8 in four), the counter-free
+// exchange 1 us less (9.4 in two slices).
 MidPlan plan_mid(int m, int n, int k, int cus) {
     MidPlan best;
     const int G = k / kGroupK, runs = ceil_div(m, mid_max_rows_per_run());
@@ -446,7 +479,8 @@ MidPlan plan_mid(int m, int n, int k, int cus) {
             const int col_blocks = mid_column_blocks(a);
             if ((size_t)runs * col_blocks * sizeof(int) > kCounterBytes) continue;
             const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
-            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + (ks > 1 ? 1.7f * ks - 1.9f : 0.f);
+            const float exchange = ks == 1 ? 0.f : (mid_flagged(a) ? 1.7f * ks - 2.9f : 1.7f * ks - 1.9f);
+            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange;
             if (!best.ok || cost < best.cost) {
                 best.ok = true;
                 best.KS = ks;
@@ -469,6 +503,7 @@ MidArgs mid_args(const MidPlan &mp, int m, int n, int k) {
     a.GS = mp.GS;
     a.waves = mp.waves;
     a.pairs = mp.pairs;
+    a.flagged = mid_flagged(a);
     return a;
 }
 
@@ -534,7 +569,7 @@ struct WorkspaceLayout {
 };
 WorkspaceLayout workspace_layout(const GemmPlan &gp, int m, int n, int k) {
     WorkspaceLayout w{};
-    size_t off = kCounterBytes;
+    size_t off = kZeroedBytes;
     if (gp.prefill) {
         w.aext = off;
         off += prefill_aext_bytes(m, k);
@@ -543,7 +578,13 @@ WorkspaceLayout workspace_layout(const GemmPlan &gp, int m, int n, int k) {
         off += prefill_partial_bytes(m, n, gp.pf);
     } else {
         w.decode_partial = off;
-        off += gp.mid ? mid_partial_bytes(mid_args(gp.mp, m, n, k)) : gp.decode_partial;
+        if (gp.mid) {
+            const MidArgs ma = mid_args(gp.mp, m, n, k);
+            if (ma.flagged) w.decode_partial = kCounterBytes;  // in the zeroed region, nothing behind it
+            else off += mid_partial_bytes(ma);
+        } else {
+            off += gp.decode_partial;
+        }
     }
     w.plain = off;
     off = (off + 255) & ~(size_t)255;
@@ -721,6 +762,8 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         a.regs = l.plan.regs;
         a.gm_tiles = l.plan.gm_tiles;
         a.gmp = l.plan.gmp;
+        a.flagged = launch_flagged(l, prob_n);
+        a.partial = reinterpret_cast<float *>(ws + (a.flagged ? kCounterBytes : wl.decode_partial));
         a.group_major = g_tune.decode_group_major;
         if ((a.gmp ? launch_decode_gmp(a, st) : launch_decode(a, st)) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
     }
@@ -737,7 +780,7 @@ size_t kiln_w4a16_workspace_bytes(int prob_m, int prob_n, int prob_k) {
 }
 
 size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k, int thread_k, int thread_n, int sms) {
-    if (prob_n <= 0 || prob_k <= 0 || !shape_ok(prob_n, prob_k, 128)) return kCounterBytes;
+    if (prob_n <= 0 || prob_k <= 0 || !shape_ok(prob_n, prob_k, 128)) return kZeroedBytes;
     int dev = 0;
     if (sms <= 0 && hipGetDevice(&dev) != hipSuccess) dev = -1;  // no device: the part's 256 units
     const int cus = sms > 0 ? sms : compute_units(dev);
@@ -745,7 +788,7 @@ size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k, int 
                                 thread_n > 0 ? thread_n : -1);
 }
 
-size_t kiln_w4a16_workspace_zeroed_bytes(void) { return kCounterBytes; }
+size_t kiln_w4a16_workspace_zeroed_bytes(void) { return kZeroedBytes; }
 
 // ---- the GEMM for callers that cannot hand over (or allocate) a workspace ----------------------
 // The workspace of kiln_marlin_w4a16_gemm -- arrival counters and the f32 partial tiles of K-sliced
@@ -864,6 +907,7 @@ void kiln_w4a16_debug_gmp(int tiles, int waves, int kslices) {
     g_tune.gmp_ks = kslices;
     tuning_changed();
 }
+void kiln_w4a16_debug_flagged(int mode) { g_tune.flagged = mode; tuning_changed(); }
 void kiln_w4a16_debug_mid(int mode, int pairs, int kslices) {
     g_tune.mid = mode;
     g_tune.mid_pairs = pairs;
@@ -923,7 +967,7 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu(const void *A, const void *B, void *
 }
 
 size_t kiln_w4a16_swiglu_workspace_bytes(int prob_m, int n_out, int prob_k) {
-    if (n_out <= 0 || n_out > INT32_MAX / 2) return kCounterBytes;
+    if (n_out <= 0 || n_out > INT32_MAX / 2) return kZeroedBytes;
     return kiln_w4a16_workspace_bytes(prob_m, 2 * n_out, prob_k);  // the same plans as the plain GEMM of that width
 }
 

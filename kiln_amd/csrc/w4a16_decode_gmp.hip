@@ -29,6 +29,18 @@ constexpr int kGmpSlotBytes = 16 * 256;  // one group of A: 16 rows x 128 bf16
 #ifndef KILN_GMP_HEAD
 #define KILN_GMP_HEAD 3
 #endif
+// Probe builds only (-DKILN_GMP_TIMELINE): wall-clock stamps (100 MHz) per wavefront.
+#ifdef KILN_GMP_TIMELINE
+__device__ long long *g_gmp_tl;
+#define KILN_GMP_TL(i, v) tl_[i] = (v)
+#define KILN_GMP_NOW() ((long long)__builtin_amdgcn_s_memrealtime())
+#else
+#define KILN_GMP_TL(i, v) \
+    do {                  \
+    } while (0)
+#define KILN_GMP_NOW() 0ll
+#endif
+
 constexpr int kGmpHead = KILN_GMP_HEAD;  // chunks requested ahead of the one being consumed
 constexpr int kGmpMaxChunks = 16;        // chunks per wavefront, at most (straight-line code)
 
@@ -83,6 +95,8 @@ struct GmpScheduleOf {
 };
 
 constexpr int gmp_slots(int gpw) { return gpw < 2 ? gpw : 2; }
+constexpr int kGmpFlaggedSlices = kDecodeFlaggedMaxSlices;  // most K slices the counter-free exchange takes
+constexpr int kGmpSpinLimit = 1 << 20;  // polls of the other slices' parts before the adding wavefront gives up
 
 // T tiles per block, GPW groups per wavefront (the first `full_waves` wavefronts; the others one
 // fewer), AQ = LDS-direct loads per group of A: 4 (16 rows), 2 (M <= 8) or 1 (M <= 4: rows 0...3
@@ -91,8 +105,12 @@ template <int T, int GPW, int AQ>
 __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     const uint16_t *__restrict__ A, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C, float *partial, int *counters, int M, int N, int K, int Gs, int KS, int GS,
-    int full_waves, int slot_bytes, int swiglu) {
+    int full_waves, int slot_bytes, int swiglu, int flagged, int col_shift) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
+#ifdef KILN_GMP_TIMELINE
+    long long tl_[8] = {};
+#endif
+    KILN_GMP_TL(0, KILN_GMP_NOW());
     constexpr int NS = gmp_slots(GPW);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -101,7 +119,12 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     const int G = K / kGroupK;
     const int NT = N / kTileN;
     const int ks = blockIdx.y;
-    const int tf = blockIdx.x * T;  // first tile of the block; tiles from NT on do not exist
+    // Blocks go to the eight dies round-robin by linear index.  With the counter-free exchange the
+    // column block is shifted by col_shift per slice, so that the slices of a tile sit on different
+    // dies: a device-scope store and the device-scope load that polls it are slow when they meet
+    // in one die's L2 (measured: 2...3 us per poll instead of 0.5).
+    const int col_block = (int)((blockIdx.x + ks * col_shift) % gridDim.x);
+    const int tf = col_block * T;  // first tile of the block; tiles from NT on do not exist
     const bool full = wave < full_waves;
     const int g_first = full ? wave * GPW : full_waves * GPW + (wave - full_waves) * (GPW - 1);
     const int g0 = ks * GS + g_first;  // all slices have GS groups
@@ -190,10 +213,12 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
 
     // every wavefront's partial tiles into its own piece of LDS, then tile ti = their sum in
     // wavefront (= ascending K) order, one tile per wavefront at a time
+    KILN_GMP_TL(1, KILN_GMP_NOW());
     f32x4 *slots = reinterpret_cast<f32x4 *>(mine);
 #pragma unroll
     for (int ti = 0; ti < T; ++ti) slots[ti * 64 + lane] = y[ti];
     __syncthreads();
+    KILN_GMP_TL(2, KILN_GMP_NOW());
 
     const int q4 = lane >> 4, c = lane & 15;
     const int tiles = min(T, NT - tf);
@@ -201,11 +226,70 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
         const int tt = tf + ti;
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int wv = 0; wv < nw; ++wv) sum += reinterpret_cast<const f32x4 *>(lds + wv * slot_bytes)[ti * 64 + lane];
-        if (KS > 1) {
+        if (KS > 1 && flagged) {
+            // The slices of the tile meet in a part of the workspace that is all zero between
+            // launches.  A word there is either zero (not written yet) or the complement of a
+            // partial sum's bits (a sum never has all bits set: that is a NaN whose payload no
+            // arithmetic here produces), so the data is its own arrival flag: no counter, no
+            // wait for the stores.  The last slice adds the parts; its blocks are dispatched after
+            // all others (grid y is the slice), so every block it waits for is running or done.
+            uint32_t *own = reinterpret_cast<uint32_t *>(partial) + ((size_t)ks * NT + tt) * 256 + lane * 4;
+            KILN_GMP_TL(3, KILN_GMP_NOW());
+            if (ks != KS - 1) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    __hip_atomic_store(own + i, ~__builtin_bit_cast(uint32_t, (float)sum[i]), __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                continue;
+            }
+            // up to kGmpFlaggedSlices - 1 other parts, all polled at once.  Every part is loaded once per
+            // poll: a second device-scope load of an address the wavefront has just loaded waits for
+            // the first (measured: 0.5 us per repeat).
+            uint32_t got[kGmpFlaggedSlices - 1][4] = {};
+            const uint32_t *base = reinterpret_cast<const uint32_t *>(partial) + (size_t)tt * 256 + lane * 4;
+            for (int spins = 0;; ++spins) {
+                bool missing = false;
+#pragma unroll
+                for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2) {
+                    if (s2 < KS - 1) {
+                        const uint32_t *src = base + (size_t)s2 * NT * 256;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            got[s2][i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+#pragma unroll
+                for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2)  // after all requests: one round trip per poll
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) missing |= s2 < KS - 1 && got[s2][i] == 0;
+                // the bound is never reached in a working launch; past it the words still missing read
+                // as NaN in the result
+                if (__builtin_amdgcn_ballot_w64(missing) == 0 || spins == kGmpSpinLimit) {
+                    KILN_GMP_TL(5, (long long)spins + 1);
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(2);
+            }
+            KILN_GMP_TL(4, KILN_GMP_NOW());
+            f32x4 total = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2) {
+                if (s2 < KS - 1) {  // ascending K order, this slice's own part last
+                    uint32_t *src = const_cast<uint32_t *>(base) + (size_t)s2 * NT * 256;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        total[i] += __builtin_bit_cast(float, ~got[s2][i]);
+                        __hip_atomic_store(src + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next launch
+                    }
+                }
+            }
+            sum = total + sum;
+        } else if (KS > 1) {
             // the slices of the tile meet in the workspace: store this part with device-scope
             // accesses, wait until the stores are acknowledged, count the arrival; the last to arrive
             // adds all parts in ascending K order (so the result does not depend on arrival order)
             // and leaves the counter zero
+            KILN_GMP_TL(3, KILN_GMP_NOW());
             float *dst = partial + ((size_t)ks * NT + tt) * 256 + lane * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) __hip_atomic_store(dst + i, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -214,6 +298,7 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             if (lane == 0) arrived = __hip_atomic_fetch_add(counters + tt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             arrived = __builtin_amdgcn_readfirstlane(arrived);
             if (arrived != KS - 1) continue;
+            KILN_GMP_TL(5, KILN_GMP_NOW());
             if (lane == 0) __hip_atomic_store(counters + tt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             sum = f32x4{0.f, 0.f, 0.f, 0.f};
             for (int s2 = 0; s2 < KS; ++s2) {
@@ -223,9 +308,18 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
                 for (int i = 0; i < 4; ++i) v[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 sum += v;
             }
+            KILN_GMP_TL(4, KILN_GMP_NOW());
         }
         store_tile_rows(C, N, M, 4 * q4, tt, c, sum, swiglu != 0);
     }
+#ifdef KILN_GMP_TIMELINE
+    tl_[6] = KILN_GMP_NOW();
+    tl_[7] = 1ll + blockIdx.y;
+    if (lane == 0 && g_gmp_tl) {
+        long long *o = g_gmp_tl + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 8;
+        for (int i = 0; i < 8; ++i) o[i] = tl_[i];
+    }
+#endif
 }
 
 int gmp_slot_bytes(int gpw, int tiles) {
@@ -242,7 +336,8 @@ hipError_t launch_gmp_tga(const DecodeArgs &a, hipStream_t stream) {
     const int slot = gmp_slot_bytes(GPW, T);
     w4a16_decode_gmp_kernel<T, GPW, AQ><<<dim3((NT + T - 1) / T, a.KS), a.waves * 64, a.waves * slot, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
-        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, slot, a.swiglu ? 1 : 0);
+        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, slot, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
+        a.flagged ? exchange_column_shift((NT + T - 1) / T) : 0);
     return hipGetLastError();
 }
 
@@ -292,6 +387,7 @@ bool decode_gmp_ok(const DecodeArgs &a) {
 hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream) {
     if (!decode_gmp_ok(a)) return hipErrorInvalidValue;
     if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
+    if (a.flagged && a.KS > kGmpFlaggedSlices) return hipErrorInvalidValue;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.gm_tiles) {
         case 1: return launch_gmp_t<1>(a, gpw, stream);
@@ -304,3 +400,9 @@ hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream) {
 }
 
 }  // namespace kiln
+
+#ifdef KILN_GMP_TIMELINE
+extern "C" int kiln_gmp_timeline(long long *buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(kiln::g_gmp_tl), &buf, sizeof(buf));
+}
+#endif

@@ -38,6 +38,8 @@ constexpr int kMidRows = 64;                    // rows per run
 constexpr int kMidSlotBytes = kMidRows * 256;   // one group of A: 64 rows x 128 bf16
 constexpr int kMidALoads = 16;                  // LDS-direct loads per group of A
 constexpr int kMidMaxGroups = 4;                // groups per wavefront, at most
+constexpr int kMidFlaggedSlices = kDecodeFlaggedMaxSlices;  // most K slices the counter-free exchange takes
+constexpr int kMidSpinLimit = 1 << 20;          // polls of the other slices' parts before the adding wavefront gives up
 
 // Issue order of a wavefront's loads -- A(g): 16 LDS-direct loads, B(g): NL register loads, the
 // weights D groups ahead in D + 1 register sets --
@@ -88,7 +90,7 @@ template <int TP, int GPW>
 __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
-    int GS, int full_waves, int swiglu) {
+    int GS, int full_waves, int swiglu, int flagged, int col_shift) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     __shared__ int s_last;
     const int tid = threadIdx.x;
@@ -104,7 +106,12 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const int ldc = swiglu ? N >> 1 : N;  // the fused gate/up result is half as wide
     uint16_t *__restrict__ C = C_all + (size_t)zr * ldc;
     const int ks = blockIdx.y;
-    const int tf = blockIdx.x * (2 * TP);  // first 16-column tile of the block
+    // Column block of this block.  Blocks go to the eight dies round-robin by linear index; the
+    // counter-free exchange shifts the column block by col_shift per slice so that the slices of a
+    // tile sit on different dies (a device-scope store and the device-scope load that polls it
+    // are slow when they meet in one die's L2).
+    const int cb = (int)((blockIdx.x + ks * col_shift) % gridDim.x);
+    const int tf = cb * (2 * TP);  // first 16-column tile of the block
     // the first `full_waves` wavefronts own GPW groups each, the others GPW - 1
     const bool full = wave < full_waves;
     const int g_first = full ? wave * GPW : full_waves * GPW + (wave - full_waves) * (GPW - 1);
@@ -331,9 +338,10 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                 }
         }
     };
-    float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + blockIdx.x) * (kItems * 256);
+    float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + cb) * (kItems * 256);
     const size_t slice_stride = (size_t)gridDim.x * (kItems * 256);  // floats between two K slices of a block
     f32x4 *mine = reinterpret_cast<f32x4 *>(slot);
+    [[maybe_unused]] f32x4 own[TP];  // counter-free exchange, last slice: this wavefront's sums, one per pair
     unrolled<0, (TP + 1) / 2>([&](auto phc) {
         constexpr int p0 = 2 * decltype(phc)::value, p1 = p0 + 2 < TP ? p0 + 2 : TP;
         if constexpr (p0 > 0) __syncthreads();  // the previous phase's sums have been read
@@ -346,6 +354,25 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                     mine[(((p - p0) * 2 + rb) * 4 + q) * 64 + lane] =
                         f32x4{acc[p][rb][4 * q], acc[p][rb][4 * q + 1], acc[p][rb][4 * q + 2], acc[p][rb][4 * q + 3]};
         __syncthreads();
+        if (flagged) {  // eight wavefronts: item (p0 + j) * 8 + wave for each pair j of the phase
+#pragma unroll
+            for (int j = 0; j < p1 - p0; ++j) {
+                const int item = (p0 + j) * 8 + wave;
+                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+                for (int wv = 0; wv < kMidWaves; ++wv)
+                    sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[(item - p0 * 8) * 64 + lane];
+                if (ks == KS - 1) {
+                    own[p0 + j] = sum;
+                } else {  // the complement of a sum's bits is never zero, so the part is its own arrival flag
+                    uint32_t *dst = reinterpret_cast<uint32_t *>(partial) + ks * slice_stride + item * 256 + lane * 4;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+                        __hip_atomic_store(dst + i, ~__builtin_bit_cast(uint32_t, (float)sum[i]), __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            return;
+        }
         for (int item = p0 * 8 + wave; item < p1 * 8; item += nw) {
             f32x4 sum = {0.f, 0.f, 0.f, 0.f};
             for (int wv = 0; wv < nw; ++wv)
@@ -361,6 +388,55 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         }
     });
     if (KS == 1) return;
+
+    if (flagged) {
+        // Counter-free exchange.  The parts live in a region that is all zero between launches; a
+        // written word is the complement of a sum's bits and never zero (a sum with all bits set
+        // would be a NaN whose payload no arithmetic here produces).  The last slice adds the
+        // parts; its blocks are dispatched after all others (grid y is the slice), so every block
+        // it waits for is running or done.  Each part is loaded once per poll.
+        if (ks != KS - 1) return;
+        uint32_t got[TP][kMidFlaggedSlices - 1][4] = {};
+        uint32_t *base = reinterpret_cast<uint32_t *>(partial) + wave * 256 + lane * 4;
+        for (int spins = 0;; ++spins) {
+#pragma unroll
+            for (int j = 0; j < TP; ++j)
+#pragma unroll
+                for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2)
+                    if (s2 < KS - 1) {
+                        const uint32_t *src = base + s2 * slice_stride + j * 8 * 256;
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            got[j][s2][i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+            bool missing = false;
+#pragma unroll
+            for (int j = 0; j < TP; ++j)
+#pragma unroll
+                for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) missing |= s2 < KS - 1 && got[j][s2][i] == 0;
+            // the bound is never reached in a working launch; past it the missing words read as NaN
+            if (__builtin_amdgcn_ballot_w64(missing) == 0 || spins == kMidSpinLimit) break;
+            __builtin_amdgcn_s_sleep(2);
+        }
+#pragma unroll
+        for (int j = 0; j < TP; ++j) {
+            f32x4 total = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2)
+                if (s2 < KS - 1) {  // ascending K order, this slice's own part last
+                    uint32_t *src = base + s2 * slice_stride + j * 8 * 256;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        total[i] += __builtin_bit_cast(float, ~got[j][s2][i]);
+                        __hip_atomic_store(src + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next launch
+                    }
+                }
+            store_item(total + own[j], j * 8 + wave);
+        }
+        return;
+    }
 
     // Exchange between the K slices of the block's tiles: device-scope stores, acknowledged
     // (vmcnt(0)) before the barrier that precedes the arrival count; the last block to arrive
@@ -398,7 +474,8 @@ hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
     w4a16_mid_kernel<TP, GPW><<<dim3((NT + 2 * TP - 1) / (2 * TP), a.KS, runs), a.waves * 64, a.waves * kMidSlotBytes,
                                stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
-        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0);
+        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
+        a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0);
     return hipGetLastError();
 }
 
@@ -432,6 +509,9 @@ bool mid_plan_ok(const MidArgs &a) {
     return full_waves >= 1 && full_waves <= a.waves;
 }
 
+// The counter-free exchange takes blocks of eight wavefronts (one item per wavefront and pair).
+bool mid_flagged_ok(const MidArgs &a) { return a.KS > 1 && a.KS <= kMidFlaggedSlices && a.waves == kMidWaves; }
+
 int mid_column_blocks(const MidArgs &a) { return (a.N / kTileN + 2 * a.pairs - 1) / (2 * a.pairs); }
 
 size_t mid_partial_bytes(const MidArgs &a) {
@@ -443,6 +523,7 @@ size_t mid_partial_bytes(const MidArgs &a) {
 hipError_t launch_mid(const MidArgs &a, hipStream_t stream) {
     if (!mid_plan_ok(a)) return hipErrorInvalidValue;
     if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
+    if (a.flagged && !mid_flagged_ok(a)) return hipErrorInvalidValue;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.pairs) {
         case 1: return launch_mid_t<1>(a, gpw, stream);

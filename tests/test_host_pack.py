@@ -408,16 +408,20 @@ def test_workspace_bytes_is_monotone_in_m(k, n):
 
 
 def test_workspace_is_small_where_nothing_is_exchanged():
-    """Decode calls on the projections whose plan exchanges nothing through the workspace need
-    little more than the counters and the LoRA projection scratch; the down projection's three
-    K slices need their partial tiles and no more."""
+    """Decode calls need little more than the zeroed prefix -- the counters and the region in which
+    K slices exchange their parts without counters, which is where the down projection's three
+    slices meet -- and the LoRA projection scratch."""
     L = _lib.load()
     z = L.kiln_w4a16_workspace_zeroed_bytes()
-    assert z == 64 * 1024
+    assert z == 64 * 1024 + 4 * 1024 * 1024
     for k, n in [(2560, 8192), (4096, 2560), (2560, 18432)]:
-        assert L.kiln_w4a16_workspace_bytes(16, n, k) <= z + 64 * 1024, (k, n)
+        assert z <= L.kiln_w4a16_workspace_bytes(16, n, k) <= z + 64 * 1024, (k, n)
+    # a call with adapters takes the kernels whose three slices meet through counters: their partial tiles
     down = L.kiln_w4a16_workspace_bytes(16, 2560, 9216)
     assert z + 3 * 2 * 2560 * 64 <= down <= z + 3 * 2 * 2560 * 64 + 64 * 1024
+    # no shape, however small or unsupported, is sized below the prefix a caller zero-fills
+    for m, n, k in [(1, 256, 128), (0, 256, 128), (16, 100, 128), (16, 256, 100)]:
+        assert L.kiln_w4a16_workspace_bytes(m, n, k) >= z
 
 
 def test_shipped_library_has_no_tuning_setters():
