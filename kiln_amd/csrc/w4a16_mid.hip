@@ -341,6 +341,13 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + cb) * (kItems * 256);
     const size_t slice_stride = (size_t)gridDim.x * (kItems * 256);  // floats between two K slices of a block
     f32x4 *mine = reinterpret_cast<f32x4 *>(slot);
+    // item `local` of the phase, summed over the wavefronts in wavefront (= ascending K) order
+    auto sum_over_wavefronts = [&](int local) {
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int wv = 0; wv < nw; ++wv)
+            sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[local * 64 + lane];
+        return sum;
+    };
     [[maybe_unused]] f32x4 own[TP];  // counter-free exchange, last slice: this wavefront's sums, one per pair
     unrolled<0, (TP + 1) / 2>([&](auto phc) {
         constexpr int p0 = 2 * decltype(phc)::value, p1 = p0 + 2 < TP ? p0 + 2 : TP;
@@ -358,9 +365,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
 #pragma unroll
             for (int j = 0; j < p1 - p0; ++j) {
                 const int item = (p0 + j) * 8 + wave;
-                f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-                for (int wv = 0; wv < kMidWaves; ++wv)
-                    sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[(item - p0 * 8) * 64 + lane];
+                const f32x4 sum = sum_over_wavefronts(item - p0 * 8);
                 if (ks == KS - 1) {
                     own[p0 + j] = sum;
                 } else {  // the complement of a sum's bits is never zero, so the part is its own arrival flag
@@ -374,9 +379,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             return;
         }
         for (int item = p0 * 8 + wave; item < p1 * 8; item += nw) {
-            f32x4 sum = {0.f, 0.f, 0.f, 0.f};
-            for (int wv = 0; wv < nw; ++wv)
-                sum += reinterpret_cast<const f32x4 *>(lds + wv * kMidSlotBytes)[(item - p0 * 8) * 64 + lane];
+            const f32x4 sum = sum_over_wavefronts(item - p0 * 8);
             if (KS == 1) {
                 store_item(sum, item);
             } else {

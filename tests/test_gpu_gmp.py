@@ -90,3 +90,30 @@ def test_private_staging_k_slices_are_deterministic_and_one_hot_exact(oracle):
         y = marlin_gemm.marlin_w4a16_gemm(bf16_tensor(oracle.np_f32_to_bf16(xh)), bt, st, 128)
         want = oracle.np_f32_to_bf16(oracle.c_dequant_f32(q, s_bits, 128)[rows])
         assert np.array_equal(bf16_bits(y), want)
+
+
+@pytest.mark.parametrize("tiles,waves,gs,n", [(1, 12, 48, 2560), (1, 12, 72, 2560), (2, 12, 48, 1024), (1, 12, 36, 512)])
+def test_private_staging_slot_reuse_is_ordered(oracle, tiles, waves, gs, n):
+    """Three and more groups per wavefront reuse the two staging slots: the request that refills a
+    slot must come after the reads of its previous occupant have completed, not merely been
+    issued.  Checked where a violation showed (first rows of a group overwritten early): on the
+    first launch after fresh uploads against the oracle, then over 2000 launches bit for bit."""
+    L = _lib.load_tuning()
+    k, m = 128 * gs, 16
+    x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=gs + n)
+    b, s = pack.repack_gptq(q, s_bits, None, 128)
+    L.kiln_w4a16_debug_gmp(tiles, waves, 1)
+    assert _plan(L, m, n, k)[7] == -tiles
+    _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
+    bt, st = upload_packed(b, s)
+    xt = bf16_tensor(x)
+    first = marlin_gemm.marlin_w4a16_gemm(xt, bt, st, 128).clone()
+    out = torch.empty_like(first)
+    same = torch.ones((), dtype=torch.bool, device=first.device)
+    for i in range(2000):
+        if i % 100 == 0:
+            bt, st = upload_packed(b, s)                     # fresh copies: cold lines, as on a first call
+            xt = bf16_tensor(x)
+        marlin_gemm.marlin_w4a16_gemm(xt, bt, st, 128, out=out)
+        same &= (out == first).all()
+    assert bool(same)
