@@ -59,7 +59,7 @@ typedef int kiln_marlin_status_t;
  *   - B and s are in the tile layout;
  *   - `workspace` must hold kiln_w4a16_workspace_bytes(m, n, k) bytes (with overrides:
  *     kiln_w4a16_workspace_bytes_tuned), its first kiln_w4a16_workspace_zeroed_bytes()
- *     bytes zero on first use; every call leaves that counter region zero again (the
+ *     bytes zero on first use; every call leaves that prefix zero again (the
  *     reference's lock array has the same in/out contract, marlin_kernel.cu:177-180);
  *   - `stream` is a hipStream_t; thread_k (rows of K per block or K slice) and
  *     thread_n (columns per block) keep the reference's meaning as overrides of
@@ -79,9 +79,11 @@ kiln_marlin_status_t kiln_marlin_w4a16_gemm(
  * reference wrapper's fixed `(n / 128) * max_par` int32 sizing (lib.rs:176-178).
  * The value is the largest need of any row count from 1 to prob_m, so it never decreases
  * with prob_m: one workspace sized for the largest m a caller will issue serves every
- * smaller call.  Only the first kiln_w4a16_workspace_zeroed_bytes() bytes (arrival
- * counters) must be zero before the first call; every call leaves them zero again, and
- * nothing else in the workspace carries state from one call to the next.
+ * smaller call, and it is never below kiln_w4a16_workspace_zeroed_bytes().  Only that prefix
+ * (arrival counters, and the region in which K slices exchange partial tiles that are their
+ * own arrival flags) must be zero before the first call; every call leaves it zero again, and
+ * nothing else in the workspace carries state from one call to the next.  A caller that
+ * overwrites the prefix between calls must zero it again before the next one.
  */
 size_t kiln_w4a16_workspace_bytes(int prob_m, int prob_n, int prob_k);
 
@@ -90,8 +92,9 @@ size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k,
                                         int thread_k, int thread_n, int sms);
 
 /*
- * Length of the workspace prefix that must be zero on first use (64 KiB of counters; the
- * reference's whole lock array has that contract, marlin_kernel.cu:177-180, lib.rs:176-178).
+ * Length of the workspace prefix that must be zero on first use (64 KiB of counters + 4 MiB in
+ * which K slices meet without counters; the reference's whole lock array has that contract,
+ * marlin_kernel.cu:177-180, lib.rs:176-178).
  */
 size_t kiln_w4a16_workspace_zeroed_bytes(void);
 
@@ -100,10 +103,10 @@ size_t kiln_w4a16_workspace_zeroed_bytes(void);
  * device memory or hand a workspace over: code running under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc.  No counterpart in the reference (its wrapper
  * allocates and zero-fills a workspace per call, lib.rs:174-178).  The counters and f32 partial
- * tiles live in a device array inside the library, KILN_W4A16_STATIC_SCRATCH_BYTES = 4 MiB per
+ * tiles live in a device array inside the library, KILN_W4A16_STATIC_SCRATCH_BYTES = 8 MiB per
  * GPU the library runs on, held until the process ends.  The call allocates nothing and frees
  * nothing.  A shape whose plan needs more than that (kiln_w4a16_workspace_bytes says how much a
- * shape needs; every decode call of the model's projections, m <= 80, needs at most 2.3 MB; large
+ * shape needs; every call of the model's projections with m <= 128 fits; large
  * K-sliced prefill calls need tens of MB) is refused with KILN_W4A16_ERR_SCRATCH before anything
  * is launched.  `dev` must be the current device.  All calls on one GPU share that GPU's array:
  * calls that may overlap in time (different streams, or threads launching concurrently) race on
