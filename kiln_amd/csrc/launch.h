@@ -45,6 +45,15 @@ struct DecodeArgs {
     int r_total = 0;               // <= 64
     int lora_slices = 1;
     int lora_rows = 0;             // rows of the whole projection (>= M: the slab may be a part of it)
+    // private-staging instance only: the projection computed inside the launch by lora_producers extra blocks
+    // (0: lora_t was written by a launch of its own).  lora_t is then written here, [lora_producers][M][rp].
+    int lora_producers = 0;        // = lora_slices, <= 16
+    int lora_steps_per_slice = 0;  // 32-value steps of K per producer
+    const void *lora_a = nullptr;  // bf16 [r_total, K]
+    unsigned *lora_flags = nullptr;  // 17 words, zero between launches
+    int lora_adapters = 0;         // 1...4
+    int lora_ends[4] = {};         // exclusive end column of adapter i (r_total past the last adapter)
+    float lora_scales[4] = {};     // its scale (0 past the last)
     bool swiglu = false;  // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
     int group_major = -1; // tuning: 0 never a group-major instance, 1 only the LDS-staged one, 2 the
                           // register-fragment one wherever a plan fits it; -1: automatic
@@ -76,6 +85,7 @@ bool decode_group_major_regs_ok(const struct DecodeArgs &a);  // ... and the one
 int decode_max_tiles_per_block();
 hipError_t launch_decode(const DecodeArgs &args, hipStream_t stream);
 bool decode_gmp_ok(const DecodeArgs &a);                        // does the plan fit the private-staging instance?
+bool decode_gmp_fold_ok(const DecodeArgs &a);                   // ... with the LoRA projection folded into the launch?
 hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream);
 
 // One launch of the mid-M kernel: runs of up to 64 rows (grid z) against the whole weight.
@@ -132,6 +142,7 @@ struct PrefillArgs {
 size_t prefill_aext_bytes(int m, int k);
 size_t prefill_lora_t_bytes(int m, bool few_rows);  // scratch of the LoRA projection on either path
 int prefill_lora_max_slices(int m);
+int lora_project_slices(int m, int k);  // K slices of the few-rows projection (before rounding to whole groups)
 struct PrefillPlan {
     int bn = 128;     // block columns
     int bm = 256;     // block rows

@@ -19,6 +19,9 @@ constexpr size_t kCounterBytes = 64 * 1024;   // arrival counters at the start o
 // wavefront that adds a tile's parts writes zeros back), and a written word is never zero.
 constexpr size_t kFlaggedBytes = 4 * 1024 * 1024;
 constexpr size_t kZeroedBytes = kCounterBytes + kFlaggedBytes;
+// the last words of that region: producer flags and reader count of a LoRA projection folded into its GEMM launch
+constexpr size_t kFoldFlagBytes = 4096;
+constexpr size_t kFoldFlagOffset = kCounterBytes + kFlaggedBytes - kFoldFlagBytes;
 
 struct DeviceInfo {
     std::once_flag once;
@@ -71,6 +74,7 @@ struct Tuning {
     int mid = -1;                     // 0 = never the mid-M kernel, 1 = wherever a plan fits (any row count), -1 = automatic
     int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
     int flagged = -1;                 // 0 = K slices always meet through counters, -1 = automatic
+    int lora_fold = -1;               // 0 = the LoRA projection always runs as a launch of its own, -1 = automatic
 };
 #ifdef KILN_W4A16_TUNING_HOOKS
 Tuning g_tune;
@@ -213,7 +217,9 @@ bool plan_decode(int n, int k, int cus, int thread_k, int thread_n, DecodeMode m
 // 17 <= m <= 32: only the register-fragment instance takes that many rows; false if no plan fits.
 constexpr long kRegsHandicap = 8;
 // the private-staging group-major instance with a given plan, if the shape takes it
-bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, DecodePlan *plan) {
+// lora: the plan must also hold for a call with adapters, whatever their ranks (one wavefront more per
+// block and the low-rank term's operands in LDS: checked for the largest rank and slice count)
+bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, bool lora, DecodePlan *plan) {
     const int G = k / kGroupK, NT = n / kTileN;
     if (ks < 1 || G % ks != 0 || tiles < 1) return false;
     DecodeArgs a;
@@ -224,6 +230,13 @@ bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, DecodePlan *pla
     a.GS = G / ks;
     a.waves = waves < a.GS ? waves : a.GS;
     a.gm_tiles = tiles;
+    if (lora) {
+        static const uint16_t probe = 0;  // never dereferenced: the check only asks for non-null operands
+        a.r_total = 64;
+        a.lora_slices = 16;
+        a.lora_rows = m;
+        a.lora_t = a.lora_b = &probe;
+    }
     if (!decode_gmp_ok(a)) return false;
     *plan = DecodePlan{};
     plan->KS = ks;
@@ -240,7 +253,7 @@ bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, DecodePlan *pla
 // but the last writes there)?
 bool flagged_exchange_fits(int ks, int n) {
     return g_tune.flagged != 0 && ks > 1 && ks <= kDecodeFlaggedMaxSlices &&
-           (size_t)(ks - 1) * (n / kTileN) * 256 * sizeof(float) <= kFlaggedBytes;
+           (size_t)(ks - 1) * (n / kTileN) * 256 * sizeof(float) <= kFlaggedBytes - kFoldFlagBytes;
 }
 
 // Best plan for the private-staging group-major instance (m <= 16).  Cost in microseconds, fitted
@@ -252,7 +265,7 @@ bool flagged_exchange_fits(int ks, int n) {
 // between K slices is priced where the cost is formed (down projection at 16 rows in three
 // slices: 7.1 us with the parts as their own arrival flags, 8.4 through counters; four, six, eight
 // slices through counters 9.2, 9.9, 11.2).
-bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
+bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) {
     const int G = k / kGroupK, NT = n / kTileN;
     const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
     static const int kWaves[] = {12, 16, 8};
@@ -266,7 +279,7 @@ bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
                 // (out-projection: 4.9 against 5.3 us with 12); elsewhere they measured slower
                 if (waves == 16 && (T != 1 || GS % 16 != 0)) continue;
                 DecodePlan p;
-                if (!gmp_plan(m, n, k, T, waves, ks, &p)) continue;
+                if (!gmp_plan(m, n, k, T, waves, ks, lora, &p)) continue;
                 const int rounds = ceil_div(ceil_div(NT, T) * ks, cus);
                 // The exchange: through counters 0.4 us per slice + 1.2; with the parts as their own
                 // arrival flags it grows with the tiles polled, 0.0037 us per (slice - 1) and tile
@@ -289,15 +302,18 @@ bool plan_decode_gmp(int m, int n, int k, int cus, DecodePlan *best) {
     return best_cost >= 0.f;
 }
 
-bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, bool lora, DecodePlan *plan,
+// lora: 0 = a call without adapters, 1 = with adapters the private-staging kernel takes (stacked rank a
+// multiple of 8), 2 = with other adapters
+bool choose_decode(int m, int n, int k, int cus, int thread_k, int thread_n, int lora, DecodePlan *plan,
                    bool *direct) {
     *direct = false;
-    if (g_tune.gmp_tiles > 0 && m <= 16 && gmp_plan(m, n, k, g_tune.gmp_tiles, g_tune.gmp_waves, g_tune.gmp_ks, plan))
+    if (g_tune.gmp_tiles > 0 && m <= 16 && lora != 2 &&
+        gmp_plan(m, n, k, g_tune.gmp_tiles, g_tune.gmp_waves, g_tune.gmp_ks, lora != 0, plan))
         return true;
-    // up to 16 rows of a call without adapters or overrides: the private-staging instance
-    if (m <= 16 && !lora && thread_k <= 0 && thread_n <= 0 && g_tune.gmp_tiles == 0 && g_tune.decode_group_major == -1 &&
+    // up to 16 rows of a call without overrides (with or without adapters): the private-staging instance
+    if (m <= 16 && lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.gmp_tiles == 0 && g_tune.decode_group_major == -1 &&
         g_tune.decode_direct_max_m < 0 && !g_tune.force_ks && !g_tune.force_u && !g_tune.force_waves &&
-        plan_decode_gmp(m, n, k, cus, plan))
+        plan_decode_gmp(m, n, k, cus, lora != 0, plan))
         return true;
     const bool regs_allowed = g_tune.decode_group_major != 0 && g_tune.decode_group_major != 1 && thread_n <= 0;
     if (m > 16) return regs_allowed && plan_decode(n, k, cus, thread_k, thread_n, DecodeMode::kRegs, m, plan);
@@ -346,8 +362,8 @@ struct SlabChoice {
 std::mutex g_plan_mutex;
 std::unordered_map<SlabKey, SlabChoice, SlabKeyHash> g_plan_cache;
 
-SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n, bool lora) {
-    const SlabKey key{m, n, k, cus, thread_k, thread_n, lora ? 1 : 0};
+SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n, int lora) {
+    const SlabKey key{m, n, k, cus, thread_k, thread_n, lora};
     {
         std::lock_guard<std::mutex> lock(g_plan_mutex);
         auto it = g_plan_cache.find(key);
@@ -449,7 +465,7 @@ constexpr int kMidMinM = 33, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN =
 
 // Do the K slices of this mid-M launch meet in the zeroed region, the parts being their own arrival flags?
 bool mid_flagged(const MidArgs &a) {
-    return g_tune.flagged != 0 && mid_flagged_ok(a) && mid_partial_bytes(a) <= kFlaggedBytes;
+    return g_tune.flagged != 0 && mid_flagged_ok(a) && mid_partial_bytes(a) <= kFlaggedBytes - kFoldFlagBytes;
 }
 
 // Plan for the mid-M kernel: pairs of tiles per block, K slices, wavefronts.  Cost in microseconds,
@@ -507,7 +523,7 @@ MidArgs mid_args(const MidPlan &mp, int m, int n, int k) {
     return a;
 }
 
-void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, bool lora, GemmPlan *gp) {
+void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lora, GemmPlan *gp) {
     *gp = GemmPlan{};
     // 33...128 rows of a plain GEMM: the mid-M kernel, one pass over the weights per 64 rows
     if (!lora && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
@@ -528,6 +544,8 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, bool lo
     // 16-row slabs in one pass over the weights; where more than 32 rows are left and that
     // instance runs, up to four runs of 32 share one launch (a later run's blocks fill the units the
     // earlier ones leave idle; each run has its own counters and partial tiles).
+    // the private-staging kernel takes adapters only where one launch covers the whole call (it reads T whole)
+    const int slab_lora = (lora == 1 && m > 16) ? 2 : lora;
     for (int r0 = 0; r0 < m;) {
         if (gp->launches == kMaxDecodeLaunches) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
         DecodeLaunch &l = gp->dl[gp->launches];
@@ -535,10 +553,10 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, bool lo
         l.r0 = r0;
         l.M = left < 32 ? left : 32;
         SlabChoice c;
-        if (l.M > 16) c = slab_choice(l.M, n, k, cus, thread_k, thread_n, lora);
+        if (l.M > 16) c = slab_choice(l.M, n, k, cus, thread_k, thread_n, slab_lora);
         if (!c.ok) {
             l.M = left < 16 ? left : 16;
-            c = slab_choice(l.M, n, k, cus, thread_k, thread_n, lora);
+            c = slab_choice(l.M, n, k, cus, thread_k, thread_n, slab_lora);
             // no small-M plan (K beyond eight slices of 32 groups): the matrix-core kernel takes any M
             if (!c.ok) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
         }
@@ -638,9 +656,9 @@ struct LoraSpec {
 size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thread_n) {
     size_t most = 0;
     auto consider = [&](int mm) {
-        for (int lora = 0; lora < 2; ++lora) {  // a call with adapters may take another path
+        for (int lora = 0; lora < 3; ++lora) {  // a call with adapters may take another path
             GemmPlan gp;
-            plan_gemm(mm, n, k, cus, thread_k, thread_n, lora != 0, &gp);
+            plan_gemm(mm, n, k, cus, thread_k, thread_n, lora, &gp);
             const size_t need = workspace_layout(gp, mm, n, k).total;
             if (need > most) most = need;
         }
@@ -667,7 +685,8 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     const int cus = sms > 0 ? sms : compute_units(dev);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     GemmPlan gp;
-    plan_gemm(prob_m, prob_n, prob_k, cus, thread_k, thread_n, lora != nullptr, &gp);
+    const int lora_kind = !lora ? 0 : (lora->r_total % 8 == 0 ? 1 : 2);
+    plan_gemm(prob_m, prob_n, prob_k, cus, thread_k, thread_n, lora_kind, &gp);
     const WorkspaceLayout wl = workspace_layout(gp, prob_m, prob_n, prob_k);
     char *ws = reinterpret_cast<char *>(workspace);
     char *lora_t = ws + wl.lora_t;
@@ -716,7 +735,38 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     }
 
     int rp = 0, lora_slices = 1;
-    if (lora) {  // the scaled projection of all rows onto the adapters, once, ahead of the runs
+    // Up to 16 rows on the private-staging kernel: the projection rides in the GEMM launch (extra
+    // blocks at the front of its grid) instead of running as a launch of its own.
+    DecodeArgs fold_probe;
+    bool fold = false;
+    int fold_steps = 0;
+    if (lora && g_tune.lora_fold != 0 && gp.launches == 1 && gp.dl[0].plan.gmp && gp.dl[0].M == prob_m) {
+        const int steps = prob_k / 32;
+        int kz = lora_project_slices(prob_m, prob_k);
+        fold_steps = ((steps + kz - 1) / kz + 3) / 4 * 4;  // whole 128-value groups, as the projection launch cuts them
+        kz = (steps + fold_steps - 1) / fold_steps;
+        fold_probe.M = prob_m;
+        fold_probe.K = prob_k;
+        fold_probe.GS = gp.dl[0].plan.GS;
+        fold_probe.waves = gp.dl[0].plan.waves;
+        fold_probe.gm_tiles = gp.dl[0].plan.gm_tiles;
+        fold_probe.r_total = lora->r_total;
+        fold_probe.lora_a = lora->a;
+        fold_probe.lora_t = lora_t;
+        fold_probe.lora_flags = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
+        fold_probe.lora_producers = fold_probe.lora_slices = kz;
+        fold_probe.lora_steps_per_slice = fold_steps;
+        fold_probe.lora_rows = prob_m;
+        fold_probe.lora_adapters = lora->n_adapters;
+        // the producers take compute units of their own: only where the launch still fits the chip in one
+        // round (the in-projection's 256 blocks do not: 12.6 us folded against 10.6 with the launch of its own)
+        fold = decode_gmp_fold_ok(fold_probe) && gp.dl[0].plan.BPS * gp.dl[0].plan.KS + kz <= cus;
+        if (fold) {
+            lora_slices = kz;
+            rp = (lora->r_total + 15) / 16 * 16;
+        }
+    }
+    if (lora && !fold) {  // the scaled projection of all rows onto the adapters, once, ahead of the runs
         PrefillArgs pj{};
         pj.A = A;
         pj.M = prob_m;
@@ -750,6 +800,19 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             a.r_total = lora->r_total;
             a.lora_slices = lora_slices;
             a.lora_rows = prob_m;
+            if (fold) {
+                a.lora_producers = lora_slices;
+                a.lora_steps_per_slice = fold_steps;
+                a.lora_a = lora->a;
+                a.lora_flags = fold_probe.lora_flags;
+                a.lora_adapters = lora->n_adapters;
+                int end = 0;
+                for (int j = 0; j < 4; ++j) {
+                    if (j < lora->n_adapters) end += lora->ranks[j];
+                    a.lora_ends[j] = end;
+                    a.lora_scales[j] = j < lora->n_adapters ? lora->scales[j] : 0.f;
+                }
+            }
         }
         a.M = l.M;
         a.rows = l.rows;
@@ -908,6 +971,7 @@ void kiln_w4a16_debug_gmp(int tiles, int waves, int kslices) {
     tuning_changed();
 }
 void kiln_w4a16_debug_flagged(int mode) { g_tune.flagged = mode; tuning_changed(); }
+void kiln_w4a16_debug_lora_fold(int mode) { g_tune.lora_fold = mode; }
 void kiln_w4a16_debug_mid(int mode, int pairs, int kslices) {
     g_tune.mid = mode;
     g_tune.mid_pairs = pairs;

@@ -35,6 +35,7 @@
 
 #include "device_common.h"
 #include "launch.h"
+#include "lora_tail.h"
 
 // This file is compiled twice: as is for the plain kernels, and with -DKILN_DECODE_LORA=1 for the
 // instances that add the low-rank term where they store a tile (with the term behind a run-time
@@ -104,55 +105,6 @@ __device__ __forceinline__ int div_small(int a, int b) {
     q += (r >= b) ? 1 : 0;
     q -= (r < 0) ? 1 : 0;
     return q;
-}
-
-// Optional low-rank term of the result: y += T * B_cat^T, where T = bf16 [M, rp] is the scaled
-// projection of the activations onto the stacked adapters (columns r_total ... rp - 1 zero, rp a
-// multiple of 16) and B_cat = bf16 [N, r_total] (crates/kiln-model/src/lora_loader.rs:213-232,
-// added unfused at forward.rs:2932-2939).  rp == 0: none.
-struct LoraTail {
-    const uint16_t *t;
-    const uint16_t *b;
-    int r_total;
-    int rp;
-    int slices;    // T = [slices][t_rows][rp]: K slices of the projection, each rounded on its own
-    int t_rows;
-};
-
-// v = rows row0 + 4 (lane / 16) ... + 3 of column lane % 16 of tile tt, in the accumulator layout.
-[[maybe_unused]] __device__ __forceinline__ void lora_add(f32x4 &v, const LoraTail &lo, int row0, int M, int tt,
-                                                          int lane) {
-    const int kq = lane >> 4, c = lane & 15;
-    int row = row0 + c;
-    row = row < M ? row : M - 1;  // rows past M: any finite operand, the products are never stored
-    const uint16_t *tp = lo.t + (size_t)row * lo.rp;
-    const uint16_t *bp = lo.b + (size_t)(tt * kTileN + c) * lo.r_total;
-    for (int j0 = 0; j0 < lo.rp; j0 += 32) {
-        const int j8 = j0 + 8 * kq;  // this lane's 8 rank columns
-        u32x4 tb = {0u, 0u, 0u, 0u};
-        if ((lo.r_total & 7) == 0) {
-            if (j8 < lo.r_total) tb = *reinterpret_cast<const u32x4 *>(bp + j8);
-        } else {
-            uint32_t e[8];
-#pragma unroll
-            for (int i = 0; i < 8; ++i) e[i] = (j8 + i < lo.r_total) ? (uint32_t)bp[j8 + i] : 0u;
-            tb = u32x4{e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16)};
-        }
-        for (int z0 = 0; z0 < lo.slices; z0 += 8) {  // eight slices requested at a time
-            u32x4 ta[8];
-#pragma unroll
-            for (int zi = 0; zi < 8; ++zi) {
-                ta[zi] = u32x4{0u, 0u, 0u, 0u};
-                if (j8 < lo.rp && z0 + zi < lo.slices)
-                    ta[zi] = *reinterpret_cast<const u32x4 *>(tp + (size_t)(z0 + zi) * lo.t_rows * lo.rp + j8);
-            }
-#pragma unroll
-            for (int zi = 0; zi < 8; ++zi)
-                if (z0 + zi < lo.slices)
-                    v = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, ta[zi]),
-                                                                __builtin_bit_cast(bf16x8, tb), v, 0, 0, 0);
-        }
-    }
 }
 
 // U: chunks per wavefront (register array size); U <= groups per slice.
@@ -846,19 +798,6 @@ __global__ __launch_bounds__(12 * 64) void w4a16_decode_gmr_kernel(
         }
         store_tile(sum, tt, sl);
     }
-}
-
-LoraTail lora_tail(const DecodeArgs &a) {
-    LoraTail lo{};
-    if (a.r_total > 0) {
-        lo.t = (const uint16_t *)a.lora_t;
-        lo.b = (const uint16_t *)a.lora_b;
-        lo.r_total = a.r_total;
-        lo.rp = (a.r_total + 15) / 16 * 16;
-        lo.slices = a.lora_slices;
-        lo.t_rows = a.lora_rows;
-    }
-    return lo;
 }
 
 template <int T, int GPW, int SL>

@@ -17,8 +17,11 @@
 //   * K slices, where a plan still has them, meet tile by tile: the wavefront that summed a tile
 //     stores its part, waits for its own stores, counts its arrival and, if it is the last,
 //     adds the parts in slice order -- no block-wide barrier in the exchange.
+#include <cstddef>
+
 #include "async_loads.h"
 #include "launch.h"
+#include "lora_tail.h"
 
 namespace kiln {
 
@@ -98,6 +101,46 @@ constexpr int gmp_slots(int gpw) { return gpw < 2 ? gpw : 2; }
 constexpr int kGmpFlaggedSlices = kDecodeFlaggedMaxSlices;  // most K slices the counter-free exchange takes
 constexpr int kGmpSpinLimit = 1 << 20;  // polls of the other slices' parts before the adding wavefront gives up
 
+// `units` 16-byte units from global memory to LDS by one wavefront, eight requests per lane in flight.
+__device__ __forceinline__ void copy_to_lds(unsigned char *dst, const uint16_t *src, int units, int lane) {
+    const u32x4 *s = reinterpret_cast<const u32x4 *>(src);
+    u32x4 *d = reinterpret_cast<u32x4 *>(dst);
+    for (int base = 0; base < units; base += 8 * 64) {
+        u32x4 r[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int u = base + 64 * i + lane;
+            r[i] = u32x4{0u, 0u, 0u, 0u};
+            if (u < units) r[i] = s[u];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int u = base + 64 * i + lane;
+            if (u < units) d[u] = r[i];
+        }
+    }
+}
+
+// The kernel's last argument and where it sits among the arguments: the kernel reads it late, through
+// the argument segment's address (see there), so its place is spelled out as a struct with the
+// kernel's parameter list.
+struct GmpLoraArgs {
+    LoraTail lo;
+    LoraFold fold;
+};
+struct GmpKernelArgs {
+    const uint16_t *A;
+    const u32x4 *B;
+    const uint16_t *S;
+    uint16_t *C;
+    float *partial;
+    int *counters;
+    int M, N, K, Gs, KS, GS, full_waves, slot_bytes, col_shift, producers, adapter, col_blocks, nw_all, swiglu, flagged;
+    GmpLoraArgs la;
+};
+constexpr int kGmpLoraArgsOffset = (int)offsetof(GmpKernelArgs, la);
+static_assert(sizeof(GmpLoraArgs) % 4 == 0, "read word by word");
+
 // T tiles per block, GPW groups per wavefront (the first `full_waves` wavefronts; the others one
 // fewer), AQ = LDS-direct loads per group of A: 4 (16 rows), 2 (M <= 8) or 1 (M <= 4: rows 0...3
 // only; the other rows of the product are computed from whatever LDS holds and never stored).
@@ -105,25 +148,48 @@ template <int T, int GPW, int AQ>
 __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     const uint16_t *__restrict__ A, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C, float *partial, int *counters, int M, int N, int K, int Gs, int KS, int GS,
-    int full_waves, int slot_bytes, int swiglu, int flagged, int col_shift) {
+    int full_waves, int slot_bytes, int col_shift, int producers, int adapter, int col_blocks, int nw_all,
+    int swiglu, int flagged, GmpLoraArgs la) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 #ifdef KILN_GMP_TIMELINE
     long long tl_[8] = {};
 #endif
     KILN_GMP_TL(0, KILN_GMP_NOW());
+    // Everything the first requests depend on is fetched from the kernel arguments in one go: left to
+    // itself the compiler fetches what lies behind the branch below only there, one more scalar
+    // round trip (0.2 us) between the launch and the first weight request.
+    asm volatile("" : : "s"(A), "s"(B), "s"(S), "s"(M), "s"(N), "s"(K), "s"(Gs), "s"(KS), "s"(GS), "s"(full_waves),
+                 "s"(slot_bytes), "s"(col_shift), "s"(producers), "s"(adapter), "s"(col_blocks), "s"(nw_all));
     constexpr int NS = gmp_slots(GPW);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nw = blockDim.x >> 6;
+    // With adapters the block has one wavefront more than the main loop uses: it fetches what the
+    // low-rank term needs into LDS while the others stream weights.
+    const int nw = nw_all - adapter;  // nw_all = wavefronts of the block
+    const bool adapter_wave = wave == nw;  // never true without adapters
     const int G = K / kGroupK;
     const int NT = N / kTileN;
     const int ks = blockIdx.y;
+    // With adapters whose projection is folded into this launch, the first `producers` blocks of
+    // the first slice compute it (the same block indices of the other slices have nothing to do).
+    if (__builtin_expect((int)blockIdx.x < producers, 0)) {
+        if (ks == 0) lora_project_slice(A, la.fold, la.lo, M, K, blockIdx.x, lds, wave, lane, nw_all);
+#ifdef KILN_GMP_TIMELINE
+        if (ks == 0 && lane == 0 && g_gmp_tl) {
+            long long *o = g_gmp_tl + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 8;
+            o[0] = tl_[0];
+            o[6] = KILN_GMP_NOW();
+            o[7] = 100;
+        }
+#endif
+        return;
+    }
     // Blocks go to the eight dies round-robin by linear index.  With the counter-free exchange the
     // column block is shifted by col_shift per slice, so that the slices of a tile sit on different
     // dies: a device-scope store and the device-scope load that polls it are slow when they meet
     // in one die's L2 (measured: 2...3 us per poll instead of 0.5).
-    const int col_block = (int)((blockIdx.x + ks * col_shift) % gridDim.x);
+    const int col_block = (int)((blockIdx.x - producers + ks * col_shift) % col_blocks);
     const int tf = col_block * T;  // first tile of the block; tiles from NT on do not exist
     const bool full = wave < full_waves;
     const int g_first = full ? wave * GPW : full_waves * GPW + (wave - full_waves) * (GPW - 1);
@@ -214,17 +280,62 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             y[ti] += acc * f16_bits_to_f32((uint16_t)sc[set]);
         });
     };
-    if (full) run(std::integral_constant<int, GPW>{});
-    else if constexpr (GPW > 1) run(std::integral_constant<int, GPW - 1>{});
-
-    // every wavefront's partial tiles into its own piece of LDS, then tile ti = their sum in
-    // wavefront (= ascending K) order, one tile per wavefront at a time
-    KILN_GMP_TL(1, KILN_GMP_NOW());
-    f32x4 *slots = reinterpret_cast<f32x4 *>(mine);
+    if (__builtin_expect(!adapter_wave, 1)) {
+        if (full) run(std::integral_constant<int, GPW>{});
+        else if constexpr (GPW > 1) run(std::integral_constant<int, GPW - 1>{});
+        // every wavefront's partial tiles into its own piece of LDS, then tile ti = their sum in
+        // wavefront (= ascending K) order, one tile per wavefront at a time
+        KILN_GMP_TL(1, KILN_GMP_NOW());
+        f32x4 *slots = reinterpret_cast<f32x4 *>(mine);
 #pragma unroll
-    for (int ti = 0; ti < T; ++ti) slots[ti * 64 + lane] = y[ti];
+        for (int ti = 0; ti < T; ++ti) slots[ti * 64 + lane] = y[ti];
+    }
+
+    // What the low-rank term needs is read from the kernel arguments only now: as ordinary
+    // parameters these values would sit in scalar registers through the whole main loop, which
+    // already uses nearly all of them.
+    GmpLoraArgs late_args{};
+    if (__builtin_expect(adapter != 0, 0)) {  // a call without adapters does not wait for these loads
+        typedef const char __attribute__((address_space(4))) *kernarg_ptr_t;
+        typedef const uint32_t __attribute__((address_space(4))) *kernarg_words_t;
+        kernarg_ptr_t kernarg = (kernarg_ptr_t)__builtin_amdgcn_kernarg_segment_ptr();
+        asm volatile("" : "+s"(kernarg));  // opaque: nothing read through it moves above this point
+        kernarg_words_t src = (kernarg_words_t)(kernarg + kGmpLoraArgsOffset);
+        struct Words {
+            uint32_t w[sizeof(GmpLoraArgs) / 4];
+        } words;
+#pragma unroll
+        for (int i = 0; i < (int)(sizeof(GmpLoraArgs) / 4); ++i) words.w[i] = src[i];
+        late_args = __builtin_bit_cast(GmpLoraArgs, words);
+    }
+    const LoraTail &lo = late_args.lo;
+    const LoraFold &fold = late_args.fold;
+    // The low-rank term y += T * B_cat^T is added where a finished tile is stored, by the slice that
+    // finishes it.  Its operands come from LDS behind the main wavefronts' slots: the adapter
+    // wavefront copies the rows of B_cat that belong to the block's tiles at once, and T -- all of
+    // it, [slices][M][rp] -- as soon as it exists: with the projection folded into this launch, when
+    // every producer's flag is up.  All of it normally lands before the slowest main wavefront
+    // reaches the barrier, so the term costs a few LDS reads and products per tile.
+    unsigned char *lora_b_lds = lds + nw * slot_bytes;
+    unsigned char *lora_t_lds = lora_b_lds + ((T * kTileN * lo.r_total * 2 + 15) & ~15);
+    const bool adds_term = adapter != 0 && ks == KS - 1;
+    if (__builtin_expect(adapter_wave && adds_term, 0)) {
+        const int live_tiles = min(T, NT - tf);
+        copy_to_lds(lora_b_lds, lo.b + (size_t)tf * kTileN * lo.r_total, live_tiles * kTileN * lo.r_total / 8, lane);
+        if (producers > 0) {
+            KILN_GMP_TL(3, KILN_GMP_NOW());
+            lora_fold_wait(fold, lane);
+            KILN_GMP_TL(4, KILN_GMP_NOW());
+        }
+        copy_to_lds(lora_t_lds, lo.t, lo.slices * lo.t_rows * lo.rp / 8, lane);
+    }
     __syncthreads();
     KILN_GMP_TL(2, KILN_GMP_NOW());
+    if (__builtin_expect(adapter_wave, 0)) {
+        // count this block; the last one zeroes the producers' flags for the next launch
+        if (adds_term && producers > 0) lora_fold_done(fold, lane);
+        return;
+    }
 
     const int q4 = lane >> 4, c = lane & 15;
     const int tiles = min(T, NT - tf);
@@ -318,6 +429,7 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             }
             KILN_GMP_TL(4, KILN_GMP_NOW());
         }
+        if (adapter) lora_add_from_lds(sum, lo, lora_t_lds, lora_b_lds, ti, M, lane);
         store_tile_rows(C, N, M, 4 * q4, tt, c, sum, swiglu != 0);
     }
 #ifdef KILN_GMP_TIMELINE
@@ -328,6 +440,15 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
         for (int i = 0; i < 8; ++i) o[i] = tl_[i];
     }
 #endif
+}
+
+// LDS behind the main wavefronts' slots for the low-rank term: the rows of B_cat of a block's tiles
+// and T whole.
+size_t gmp_adapter_lds_bytes(const DecodeArgs &a) {
+    if (a.r_total <= 0) return 0;
+    const size_t rp = (size_t)(a.r_total + 15) / 16 * 16;
+    const size_t b_bytes = ((size_t)a.gm_tiles * kTileN * a.r_total * 2 + 15) & ~(size_t)15;
+    return b_bytes + (size_t)a.lora_slices * a.lora_rows * rp * 2;
 }
 
 int gmp_slot_bytes(int gpw, int tiles) {
@@ -342,10 +463,27 @@ hipError_t launch_gmp_tga(const DecodeArgs &a, hipStream_t stream) {
     const int NT = a.N / kTileN;
     const int full_waves = a.GS - a.waves * (GPW - 1);
     const int slot = gmp_slot_bytes(GPW, T);
-    w4a16_decode_gmp_kernel<T, GPW, AQ><<<dim3((NT + T - 1) / T, a.KS), a.waves * 64, a.waves * slot, stream>>>(
+    const int col_blocks = (NT + T - 1) / T;
+    LoraFold fold{};
+    if (a.lora_producers > 0) {
+        fold.a_cat = (const uint16_t *)a.lora_a;
+        fold.t = (uint16_t *)const_cast<void *>(a.lora_t);
+        fold.flags = a.lora_flags;
+        fold.producers = a.lora_producers;
+        fold.steps_per_slice = a.lora_steps_per_slice;
+        fold.consumers = col_blocks;
+        const int *e = a.lora_ends;
+        const float *sc = a.lora_scales;
+        fold.e0 = e[0], fold.e1 = e[1], fold.e2 = e[2], fold.e3 = e[3];
+        fold.s0 = sc[0], fold.s1 = sc[1], fold.s2 = sc[2], fold.s3 = sc[3];
+    }
+    const int grid_x = col_blocks + fold.producers;
+    const int adapter = a.r_total > 0 ? 1 : 0;  // one wavefront more: it fetches the low-rank term's operands
+    const size_t lds_bytes = (size_t)a.waves * slot + gmp_adapter_lds_bytes(a);
+    w4a16_decode_gmp_kernel<T, GPW, AQ><<<dim3(grid_x, a.KS), (a.waves + adapter) * 64, lds_bytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
-        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, slot, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
-        a.flagged ? exchange_column_shift((NT + T - 1) / T) : 0);
+        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, slot, a.flagged ? exchange_column_shift(grid_x) : 0, fold.producers,
+        adapter, col_blocks, a.waves + adapter, a.swiglu ? 1 : 0, a.flagged ? 1 : 0, GmpLoraArgs{lora_tail(a), fold});
     return hipGetLastError();
 }
 
@@ -383,19 +521,39 @@ hipError_t launch_gmp_t(const DecodeArgs &a, int gpw, hipStream_t stream) {
 // chunks each; a.waves <= 16 and <= GS.
 bool decode_gmp_ok(const DecodeArgs &a) {
     const int G = a.K / kGroupK;
-    if (a.M < 1 || a.M > 16 || a.r_total > 0 || a.gm_tiles < 1 || a.gm_tiles > 6) return false;
+    if (a.M < 1 || a.M > 16 || a.gm_tiles < 1 || a.gm_tiles > 6) return false;
+    if (a.r_total > 0) {
+        // the low-rank term has no gate/up split; its operands are read from LDS in 16-byte pieces by one
+        // wavefront more than the main loop uses; T is whole and belongs to exactly this launch's rows
+        if (a.swiglu || a.r_total > 64 || a.r_total % 8 != 0 || a.waves + 1 > kGmpMaxWaves) return false;
+        if (a.lora_slices < 1 || a.lora_slices > 16 || a.lora_rows != a.M || !a.lora_t || !a.lora_b) return false;
+    }
     if (a.KS < 1 || a.GS < 1 || a.KS * a.GS != G || a.waves < 1 || a.waves > kGmpMaxWaves || a.waves > a.GS) return false;
     const int gpw = (a.GS + a.waves - 1) / a.waves, T = a.gm_tiles;
     if (gpw > (T <= 2 ? 6 : 3) || T * gpw > kGmpMaxChunks) return false;
     const int full_waves = a.GS - a.waves * (gpw - 1);
     if (full_waves < 1 || full_waves > a.waves) return false;
-    return (size_t)a.waves * gmp_slot_bytes(gpw, T) <= (size_t)decode_max_lds_bytes();
+    return (size_t)a.waves * gmp_slot_bytes(gpw, T) + gmp_adapter_lds_bytes(a) <= (size_t)decode_max_lds_bytes();
+}
+
+// The projection folded into the launch: one producer block per K slice of it, each with at least
+// as many wavefronts as T has rank tiles and a KiB of LDS per wavefront for their meeting.
+bool decode_gmp_fold_ok(const DecodeArgs &a) {
+    if (a.r_total < 1 || a.r_total > 64 || !a.lora_a || !a.lora_t || !a.lora_flags) return false;
+    const int jt = (a.r_total + 15) / 16;
+    if (a.lora_producers < 1 || a.lora_producers > kLoraFoldMaxProducers || a.lora_producers != a.lora_slices) return false;
+    if (a.lora_steps_per_slice < 1 || (long)a.lora_producers * a.lora_steps_per_slice * 32 < a.K) return false;
+    if (a.waves < jt || (a.lora_steps_per_slice + a.waves / jt - 1) / (a.waves / jt) > kLoraFoldStepsPerWave ||
+        a.lora_rows != a.M || a.lora_adapters < 1 || a.lora_adapters > kLoraFoldMaxAdapters) return false;
+    const int gpw = (a.GS + a.waves - 1) / a.waves;
+    return gmp_slot_bytes(gpw, a.gm_tiles) >= 1024;
 }
 
 hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream) {
     if (!decode_gmp_ok(a)) return hipErrorInvalidValue;
     if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
     if (a.flagged && a.KS > kGmpFlaggedSlices) return hipErrorInvalidValue;
+    if (a.lora_producers > 0 && !decode_gmp_fold_ok(a)) return hipErrorInvalidValue;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.gm_tiles) {
         case 1: return launch_gmp_t<1>(a, gpw, stream);

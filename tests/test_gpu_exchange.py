@@ -117,3 +117,71 @@ def test_counter_free_exchange_with_nan_inf_and_zero_rows(oracle):
     out2, _ = _call(L, bf16_tensor(x2), bt, st, m, k, n, ws)
     err, _, _ = row_errors(bf16_bits(out2), oracle.c_w4a16_cpu_path(x2, q, s_bits, 128), oracle)
     assert err.max() <= 1e-2
+
+
+def _lora_call(L, xt, bt, st, la, lb, ranks, scales, m, k, n, ws=None):
+    import ctypes
+    dev = torch.cuda.current_device()
+    stream = torch.cuda.current_stream().cuda_stream
+    z = L.kiln_w4a16_workspace_zeroed_bytes()
+    if ws is None:
+        ws = torch.empty(L.kiln_w4a16_workspace_bytes(m, n, k), dtype=torch.uint8, device="cuda")
+        ws[z:].fill_(0xA5)
+        ws[:z].zero_()
+    out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+    c_ranks = (ctypes.c_int * len(ranks))(*ranks)
+    c_scales = (ctypes.c_float * len(ranks))(*scales)
+    rc = L.kiln_w4a16_gemm_lora(xt.data_ptr(), bt.data_ptr(), out.data_ptr(), st.data_ptr(), m, n, k, ws.data_ptr(),
+                                128, dev, stream, la.data_ptr(), lb.data_ptr(), sum(ranks), len(ranks), c_ranks, c_scales)
+    assert rc == _lib.OK, _lib.status_string(rc)
+    torch.cuda.synchronize()
+    assert int(ws[:z].count_nonzero()) == 0, "the call left words in the zeroed prefix"
+    return out, ws
+
+
+@pytest.mark.parametrize("m,k,n,ranks", [
+    (16, 2560, 18432, (16, 32)),        # the benchmark's adapters on gate+up
+    (4, 9216, 2560, (16, 32)),          # unsliced down projection, 15 producers
+    (16, 9216, 2560, (8,)),             # three K slices: the last one adds the term
+    (9, 4096, 2560, (64,)),             # the largest rank
+    (16, 2560, 2560, (8, 8, 8, 8)),     # four adapters
+    (16, 2560, 2560, (8, 8, 8, 8, 8)),  # five: the projection runs as a launch of its own
+    (16, 2560, 8192, (16, 32)),         # 256 column blocks: no compute unit left for producers, a launch of its own
+    (1, 256, 256, (8,)),                # two groups of K, one producer
+])
+def test_lora_projection_inside_the_gemm_launch(oracle, m, k, n, ranks):
+    """Up to 16 rows: the projection onto the adapters is computed by extra blocks of the GEMM launch,
+    which raise flags in the zeroed workspace prefix; the adding blocks' extra wavefront waits for
+    them, fetches T and the rows of B into LDS, and the last block zeroes the flags.  Against the
+    oracle with the projection folded and as a launch of its own, the prefix clean after every call,
+    a repeat on the same workspace bit-identical, and 300 launches in a row identical."""
+    L = _lib.load_tuning()
+    scales = tuple(0.5 + 0.25 * i for i in range(len(ranks)))
+    x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=300 + m + len(ranks))
+    b, s = pack.repack_gptq(q, s_bits, None, 128)
+    bt, st = upload_packed(b, s)
+    a_list = [oracle.gen_normal_bf16(r, k, 0.05, seed=60 + i) for i, r in enumerate(ranks)]
+    b_list = [oracle.gen_normal_bf16(n, r, 0.05, seed=70 + i) for i, r in enumerate(ranks)]
+    y_ref = oracle.c_w4a16_cpu_path(x, q, s_bits, 128)
+    for a_i, b_i, sc in zip(a_list, b_list, scales):
+        oracle.c_lora_delta_add(y_ref, x, a_i, b_i, sc)
+    la, lb = bf16_tensor(np.concatenate(a_list, axis=0)), bf16_tensor(np.concatenate(b_list, axis=1))
+    xt = bf16_tensor(x)
+    outs = {}
+    for fold in (-1, 0):
+        L.kiln_w4a16_debug_lora_fold(fold)
+        out, ws = _lora_call(L, xt, bt, st, la, lb, ranks, scales, m, k, n)
+        again, _ = _lora_call(L, xt, bt, st, la, lb, ranks, scales, m, k, n, ws)
+        assert torch.equal(out, again)
+        err, _, _ = row_errors(bf16_bits(out), y_ref, oracle)
+        assert err.max() <= 1e-2, (fold, err.max())
+        outs[fold] = out
+    L.kiln_w4a16_debug_lora_fold(-1)
+    same = torch.ones((), dtype=torch.bool, device="cuda")
+    out = torch.empty_like(outs[-1])
+    from kiln_amd import marlin_gemm
+    first = marlin_gemm.marlin_w4a16_gemm_lora(xt, bt, st, 128, la, lb, ranks, scales).clone()
+    for _ in range(300):
+        marlin_gemm.marlin_w4a16_gemm_lora(xt, bt, st, 128, la, lb, ranks, scales, out=out)
+        same &= (out == first).all()
+    assert bool(same) and torch.equal(first, outs[-1])

@@ -416,7 +416,8 @@ def test_workspace_is_small_where_nothing_is_exchanged():
     assert z == 64 * 1024 + 4 * 1024 * 1024
     for k, n in [(2560, 8192), (4096, 2560), (2560, 18432)]:
         assert z <= L.kiln_w4a16_workspace_bytes(16, n, k) <= z + 64 * 1024, (k, n)
-    # a call with adapters takes the kernels whose three slices meet through counters: their partial tiles
+    # adapters whose stacked rank is not a multiple of 8 take the kernels whose three slices meet through
+    # counters: their partial tiles
     down = L.kiln_w4a16_workspace_bytes(16, 2560, 9216)
     assert z + 3 * 2 * 2560 * 64 <= down <= z + 3 * 2 * 2560 * 64 + 64 * 1024
     # no shape, however small or unsupported, is sized below the prefix a caller zero-fills
