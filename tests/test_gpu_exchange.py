@@ -185,3 +185,18 @@ def test_lora_projection_inside_the_gemm_launch(oracle, m, k, n, ranks):
         marlin_gemm.marlin_w4a16_gemm_lora(xt, bt, st, 128, la, lb, ranks, scales, out=out)
         same &= (out == first).all()
     assert bool(same) and torch.equal(first, outs[-1])
+    # launches with changing activations in a row: every T must be this launch's, never an earlier one's
+    # left in some cache (two inputs alternate, each result against the oracle's for its own input)
+    x2, _, _ = oracle.gen_problem(m, k, n, 128, seed=900 + m)
+    y2_ref = oracle.c_w4a16_cpu_path(x2, q, s_bits, 128)
+    for a_i, b_i, sc in zip(a_list, b_list, scales):
+        oracle.c_lora_delta_add(y2_ref, x2, a_i, b_i, sc)
+    xt2 = bf16_tensor(x2)
+    results = []
+    for i in range(40):
+        results.append(marlin_gemm.marlin_w4a16_gemm_lora(xt2 if i % 2 else xt, bt, st, 128, la, lb, ranks, scales))
+    torch.cuda.synchronize()
+    for i, y in enumerate(results):
+        assert torch.equal(y, results[i % 2]), i
+    err, _, _ = row_errors(bf16_bits(results[1]), y2_ref, oracle)
+    assert err.max() <= 1e-2 and torch.equal(results[0], first)
