@@ -56,6 +56,15 @@ __device__ __forceinline__ void load_u16(uint32_t &dst, const void *base, uint32
     asm volatile("global_load_ushort %0, %1, %2" : "=&v"(dst) : "v"(lane_off), "s"(base) : "memory");
 }
 
+// Device-scope (coherent across the dies) 128-bit accesses: one instruction where four 32-bit
+// atomic accesses would be four.  The load is a request like the ones above: wait, then pin.
+__device__ __forceinline__ void store_b128_device_scope(void *ptr, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(v) : "memory");
+}
+__device__ __forceinline__ void load_b128_device_scope(u32x4 &dst, const void *ptr) {
+    asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(dst) : "v"(ptr) : "memory");
+}
+
 // Orders every later use of v after this point (and hence after the preceding wait).
 __device__ __forceinline__ void pin_loaded(u32x4 &v) { asm volatile("" : "+v"(v)); }
 __device__ __forceinline__ void pin_loaded(uint32_t &v) { asm volatile("" : "+v"(v)); }

@@ -250,10 +250,11 @@ bool gmp_plan(int m, int n, int k, int tiles, int waves, int ks, bool lora, Deco
 }
 
 // Can ks slices of n columns exchange their 16-row partial tiles in the zeroed region (every slice
-// but the last writes there)?
+// but the last writes there; the polling wavefront reads the parts of the largest slice count, the
+// absent ones as zeros, so the region must hold those too)?
 bool flagged_exchange_fits(int ks, int n) {
     return g_tune.flagged != 0 && ks > 1 && ks <= kDecodeFlaggedMaxSlices &&
-           (size_t)(ks - 1) * (n / kTileN) * 256 * sizeof(float) <= kFlaggedBytes - kFoldFlagBytes;
+           (size_t)(kDecodeFlaggedMaxSlices - 1) * (n / kTileN) * 256 * sizeof(float) <= kFlaggedBytes - kFoldFlagBytes;
 }
 
 // Best plan for the private-staging group-major instance (m <= 16).  Cost in microseconds, fitted

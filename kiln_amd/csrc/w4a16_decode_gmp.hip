@@ -355,32 +355,26 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             uint32_t *own = reinterpret_cast<uint32_t *>(partial) + ((size_t)ks * NT + tt) * 256 + lane * 4;
             KILN_GMP_TL(3, KILN_GMP_NOW());
             if (ks != KS - 1) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    __hip_atomic_store(own + i, ~__builtin_bit_cast(uint32_t, (float)sum[i]), __ATOMIC_RELAXED,
-                                       __HIP_MEMORY_SCOPE_AGENT);
+                const u32x4 bits = __builtin_bit_cast(u32x4, sum);
+                store_b128_device_scope(own, u32x4{~bits.x, ~bits.y, ~bits.z, ~bits.w});
                 continue;
             }
-            // up to kGmpFlaggedSlices - 1 other parts, all polled at once.  Every part is loaded once per
-            // poll: a second device-scope load of an address the wavefront has just loaded waits for
-            // the first (measured: 0.5 us per repeat).
-            uint32_t got[kGmpFlaggedSlices - 1][4] = {};
+            // The other parts, all polled at once, one 128-bit device-scope load each.  Every load of a
+            // poll goes to an address of its own -- a second device-scope load of an address the
+            // wavefront has just loaded waits for the first (measured: 0.5 us per repeat) -- so a slice
+            // index past the last other part reads the same tile in a part nobody writes (zeros).
+            u32x4 got[kGmpFlaggedSlices - 1];
             const uint32_t *base = reinterpret_cast<const uint32_t *>(partial) + (size_t)tt * 256 + lane * 4;
             for (int spins = 0;; ++spins) {
+#pragma unroll
+                for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2) load_b128_device_scope(got[s2], base + (size_t)s2 * NT * 256);
+                wait_vector_loads<0>();
                 bool missing = false;
 #pragma unroll
                 for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2) {
-                    if (s2 < KS - 1) {
-                        const uint32_t *src = base + (size_t)s2 * NT * 256;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            got[s2][i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
+                    pin_loaded(got[s2]);
+                    missing |= s2 < KS - 1 && (got[s2].x == 0 || got[s2].y == 0 || got[s2].z == 0 || got[s2].w == 0);
                 }
-#pragma unroll
-                for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2)  // after all requests: one round trip per poll
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) missing |= s2 < KS - 1 && got[s2][i] == 0;
                 // the bound is never reached in a working launch; past it the words still missing read
                 // as NaN in the result
                 if (__builtin_amdgcn_ballot_w64(missing) == 0 || spins == kGmpSpinLimit) {
@@ -394,12 +388,10 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
 #pragma unroll
             for (int s2 = 0; s2 < kGmpFlaggedSlices - 1; ++s2) {
                 if (s2 < KS - 1) {  // ascending K order, this slice's own part last
-                    uint32_t *src = const_cast<uint32_t *>(base) + (size_t)s2 * NT * 256;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        total[i] += __builtin_bit_cast(float, ~got[s2][i]);
-                        __hip_atomic_store(src + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next launch
-                    }
+                    const u32x4 g = got[s2];
+                    total += __builtin_bit_cast(f32x4, u32x4{~g.x, ~g.y, ~g.z, ~g.w});
+                    store_b128_device_scope(const_cast<uint32_t *>(base) + (size_t)s2 * NT * 256,
+                                            u32x4{0u, 0u, 0u, 0u});  // zero for the next launch
                 }
             }
             sum = total + sum;
