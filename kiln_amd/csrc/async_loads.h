@@ -58,8 +58,11 @@ __device__ __forceinline__ void load_u16(uint32_t &dst, const void *base, uint32
 
 // Device-scope (coherent across the dies) 128-bit accesses: one instruction where four 32-bit
 // atomic accesses would be four.  The load is a request like the ones above: wait, then pin.
+// A store of more than 64 bits reads the upper part of its data registers after it has issued: a
+// vector ALU instruction in the next two issue slots that overwrites them changes what is stored.
+// The compiler pads that for its own stores and cannot see into this one, hence the s_nop.
 __device__ __forceinline__ void store_b128_device_scope(void *ptr, u32x4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(ptr), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(ptr), "v"(v) : "memory");
 }
 __device__ __forceinline__ void load_b128_device_scope(u32x4 &dst, const void *ptr) {
     asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(dst) : "v"(ptr) : "memory");

@@ -466,7 +466,9 @@ constexpr int kMidMinM = 33, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN =
 
 // Do the K slices of this mid-M launch meet in the zeroed region, the parts being their own arrival flags?
 bool mid_flagged(const MidArgs &a) {
-    return g_tune.flagged != 0 && mid_flagged_ok(a) && mid_partial_bytes(a) <= kFlaggedBytes - kFoldFlagBytes;
+    // the last slice polls kMidFlaggedSlices - 1 parts whatever KS is: up to one slice's parts past the launch's own
+    return g_tune.flagged != 0 && mid_flagged_ok(a) &&
+           mid_partial_bytes(a) / a.KS * (a.KS + 1) <= kFlaggedBytes - kFoldFlagBytes;
 }
 
 // Plan for the mid-M kernel: pairs of tiles per block, K slices, wavefronts.  Cost in microseconds,

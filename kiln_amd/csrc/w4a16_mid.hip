@@ -369,11 +369,9 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                 if (ks == KS - 1) {
                     own[p0 + j] = sum;
                 } else {  // the complement of a sum's bits is never zero, so the part is its own arrival flag
-                    uint32_t *dst = reinterpret_cast<uint32_t *>(partial) + ks * slice_stride + item * 256 + lane * 4;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i)
-                        __hip_atomic_store(dst + i, ~__builtin_bit_cast(uint32_t, (float)sum[i]), __ATOMIC_RELAXED,
-                                           __HIP_MEMORY_SCOPE_AGENT);
+                    const u32x4 bits = __builtin_bit_cast(u32x4, sum);
+                    store_b128_device_scope(partial + ks * slice_stride + item * 256 + lane * 4,
+                                            u32x4{~bits.x, ~bits.y, ~bits.z, ~bits.w});
                 }
             }
             return;
@@ -383,10 +381,8 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             if (KS == 1) {
                 store_item(sum, item);
             } else {
-                float *dst = partial + ks * slice_stride + item * 256 + lane * 4;
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-                    __hip_atomic_store(dst + i, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                store_b128_device_scope(partial + ks * slice_stride + item * 256 + lane * 4,
+                                        __builtin_bit_cast(u32x4, sum));
             }
         }
     });
@@ -397,28 +393,28 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         // written word is the complement of a sum's bits and never zero (a sum with all bits set
         // would be a NaN whose payload no arithmetic here produces).  The last slice adds the
         // parts; its blocks are dispatched after all others (grid y is the slice), so every block
-        // it waits for is running or done.  Each part is loaded once per poll.
+        // it waits for is running or done.  Each part is loaded once per poll; the loads are
+        // straight-line code up to their wait, so the parts of absent slices (zeros nobody
+        // writes, or another run's parts) are loaded too and ignored.
         if (ks != KS - 1) return;
-        uint32_t got[TP][kMidFlaggedSlices - 1][4] = {};
+        u32x4 got[TP][kMidFlaggedSlices - 1] = {};
         uint32_t *base = reinterpret_cast<uint32_t *>(partial) + wave * 256 + lane * 4;
         for (int spins = 0;; ++spins) {
 #pragma unroll
             for (int j = 0; j < TP; ++j)
 #pragma unroll
                 for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2)
-                    if (s2 < KS - 1) {
-                        const uint32_t *src = base + s2 * slice_stride + j * 8 * 256;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            got[j][s2][i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
+                    load_b128_device_scope(got[j][s2], base + s2 * slice_stride + j * 8 * 256);
+            wait_vector_loads<0>();
             bool missing = false;
 #pragma unroll
             for (int j = 0; j < TP; ++j)
 #pragma unroll
-                for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2)
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) missing |= s2 < KS - 1 && got[j][s2][i] == 0;
+                for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2) {
+                    pin_loaded(got[j][s2]);
+                    const u32x4 g = got[j][s2];
+                    missing |= s2 < KS - 1 && (g.x == 0 || g.y == 0 || g.z == 0 || g.w == 0);
+                }
             // the bound is never reached in a working launch; past it the missing words read as NaN
             if (__builtin_amdgcn_ballot_w64(missing) == 0 || spins == kMidSpinLimit) break;
             __builtin_amdgcn_s_sleep(2);
@@ -429,12 +425,9 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
 #pragma unroll
             for (int s2 = 0; s2 < kMidFlaggedSlices - 1; ++s2)
                 if (s2 < KS - 1) {  // ascending K order, this slice's own part last
-                    uint32_t *src = base + s2 * slice_stride + j * 8 * 256;
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        total[i] += __builtin_bit_cast(float, ~got[j][s2][i]);
-                        __hip_atomic_store(src + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // zero for the next launch
-                    }
+                    const u32x4 g = got[j][s2];
+                    total += __builtin_bit_cast(f32x4, u32x4{~g.x, ~g.y, ~g.z, ~g.w});
+                    store_b128_device_scope(base + s2 * slice_stride + j * 8 * 256, u32x4{0, 0, 0, 0});  // zero for the next launch
                 }
             store_item(total + own[j], j * 8 + wave);
         }
@@ -457,11 +450,11 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     for (int item = wave; item < kItems; item += nw) {
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int s2 = 0; s2 < KS; ++s2) {
-            const float *src = partial + s2 * slice_stride + item * 256 + lane * 4;
-            f32x4 v;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) v[i] = __hip_atomic_load(src + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            sum += v;
+            u32x4 v;
+            load_b128_device_scope(v, partial + s2 * slice_stride + item * 256 + lane * 4);
+            wait_vector_loads<0>();
+            pin_loaded(v);
+            sum += __builtin_bit_cast(f32x4, v);
         }
         store_item(sum, item);
     }
