@@ -265,9 +265,11 @@ bool flagged_exchange_fits(int ks, int n) {
 // and not at 4 rows; a wavefront's chunks run one after the other (0.08 us each); the exchange
 // between K slices is priced where the cost is formed (down projection at 16 rows in three
 // slices: 7.1 us with the parts as their own arrival flags, 8.4 through counters; four, six, eight
-// slices through counters 9.2, 9.9, 11.2).
+// slices through counters 9.2, 9.9, 11.2).  A call with adapters plans for the chip less the blocks
+// that project x onto the adapters, so that the projection can ride in the same launch.
 bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) {
     const int G = k / kGroupK, NT = n / kTileN;
+    if (lora && g_tune.lora_fold != 0) cus -= lora_project_slices(m, k);
     const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
     static const int kWaves[] = {12, 16, 8};
     float best_cost = -1.f;
@@ -285,7 +287,8 @@ bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) 
                 // The exchange: through counters 0.4 us per slice + 1.2; with the parts as their own
                 // arrival flags it grows with the tiles polled, 0.0037 us per (slice - 1) and tile
                 // (down projection, 160 tiles: 0.4 / 1.1 / 1.9 us at two / three / four slices;
-                // in-projection, 512 tiles: 2.0 us at two), + 0.3 because the unsliced estimates
+                // in-projection, 512 tiles: 2.0 us at two; 576 tiles in two slices of five-tile
+                // blocks: 7.0 us against 6.1 unsliced), + 0.3 because the unsliced estimates
                 // run high.  At up to four rows the additive model puts sliced plans 1 us too low
                 // (down projection: 6.7 us in three slices against 5.7 unsliced): + 0.7 there.
                 const bool flagged = flagged_exchange_fits(ks, n);
