@@ -33,6 +33,16 @@ namespace kiln {
 
 namespace {
 
+// Probe builds only (-DKILN_MID_TIMELINE): wall-clock stamps (100 MHz) per wavefront.
+#ifdef KILN_MID_TIMELINE
+__device__ long long *g_mid_tl;
+#define KILN_MID_TL(i) tl_[i] = (long long)__builtin_amdgcn_s_memrealtime()
+#else
+#define KILN_MID_TL(i) \
+    do {               \
+    } while (0)
+#endif
+
 constexpr int kMidWaves = 8;                    // wavefronts per block, at most
 constexpr int kMidRows = 64;                    // rows per run
 constexpr int kMidSlotBytes = kMidRows * 256;   // one group of A: 64 rows x 128 bf16
@@ -43,7 +53,9 @@ constexpr int kMidSpinLimit = 1 << 20;          // polls of the other slices' pa
 
 // Issue order of a wavefront's loads -- A(g): 16 LDS-direct loads, B(g): NL register loads, the
 // weights D groups ahead in D + 1 register sets --
-//   before the first step: A(0), B(0) ... B(D-1);
+//   before the first step: A(0), B(0) ... B(D-1) (the weights first measured 0.3...0.5 us slower:
+//     loads return in issue order, so A(0) then waits for the weights' trip to memory before the
+//     fragments can be read and A(1) asked for);
 //   step g: [wait for A(g)] fragments to registers, A(g+1), B(g+D), [wait for B(g)], products.
 // wait_a[g] / wait_b[g] = loads issued after A(g) / B(g) up to that wait: what may still be
 // outstanding when the wait returns.
@@ -99,6 +111,21 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const int nw = blockDim.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int G = K / kGroupK;
+#ifdef KILN_MID_TIMELINE
+    long long tl_[8] = {};
+    struct TimelineWriter {  // on every way out of the kernel
+        long long *tl;
+        int lane, wave;
+        __device__ ~TimelineWriter() {
+            tl[7] = (long long)__builtin_amdgcn_s_memrealtime();
+            if (lane == 0 && g_mid_tl) {
+                long long *o = g_mid_tl + ((((size_t)blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x) * 8 + wave) * 8;
+                for (int i = 0; i < 8; ++i) o[i] = tl[i];
+            }
+        }
+    } timeline_writer{tl_, lane, wave};
+#endif
+    KILN_MID_TL(0);
     // blockIdx.z: which run of 64 rows (each with its own counters and partial tiles)
     const int zr = blockIdx.z * kMidRows;
     const int M = min(rows - zr, kMidRows);
@@ -193,7 +220,10 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             constexpr int gi = decltype(gc)::value, set = gi % kSets;
             // this group's rows of A are in LDS; their fragments go to registers: lane (l32, h) holds
             // row 32 rb + l32, values 16 s + 8 h ... + 7 of the group
+            if constexpr (gi == 1) KILN_MID_TL(3);  // products of group 0 issued
             wait_vector_loads<Sch::value.wait_a[gi]>();
+            if constexpr (gi == 0) KILN_MID_TL(1);  // A(0) has arrived
+            if constexpr (gi == 1) KILN_MID_TL(4);  // A(1) has arrived
             u32x4 af[2][8];
 #pragma unroll
             for (int rb = 0; rb < 2; ++rb)
@@ -229,6 +259,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                 c_of[gi][rb] = -kCodeBias * (half_sum + __shfl_xor(half_sum, 32, 64));
             }
             wait_vector_loads<Sch::value.wait_b[gi]>();
+            if constexpr (gi == 0) KILN_MID_TL(2);  // B(0) has arrived
 #pragma unroll
             for (int p = 0; p < TP; ++p) {
                 pin_loaded(bw[set][p][0]);
@@ -301,6 +332,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     };
     if (full) run(std::integral_constant<int, GPW>{});
     else if constexpr (GPW > 1) run(std::integral_constant<int, GPW - 1>{});
+    KILN_MID_TL(5);  // main loop done
 
     // --- the wavefronts' partial tiles meet in LDS, at most two pairs at a time (a wavefront's
     // 16 KiB slot holds two pairs' tiles): every wavefront writes its own slot (item = (pair, row
@@ -361,6 +393,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                     mine[(((p - p0) * 2 + rb) * 4 + q) * 64 + lane] =
                         f32x4{acc[p][rb][4 * q], acc[p][rb][4 * q + 1], acc[p][rb][4 * q + 2], acc[p][rb][4 * q + 3]};
         __syncthreads();
+        if constexpr (p0 == 0) KILN_MID_TL(6);  // every wavefront's tiles are in LDS
         if (flagged) {  // eight wavefronts: item (p0 + j) * 8 + wave for each pair j of the phase
 #pragma unroll
             for (int j = 0; j < p1 - p0; ++j) {
@@ -529,3 +562,9 @@ hipError_t launch_mid(const MidArgs &a, hipStream_t stream) {
 }
 
 }  // namespace kiln
+
+#ifdef KILN_MID_TIMELINE
+extern "C" int kiln_mid_timeline(long long *buf) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(kiln::g_mid_tl), &buf, sizeof(buf));
+}
+#endif
