@@ -35,8 +35,8 @@ GROUP = 128
 LAYERS = 16
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
-# copy (x1.9989 and x1.0): 12289.9 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
-GATE_UP_M16_TRAFFIC_BYTES = 25745700
+# copy (x1.9989 and x1.0): 12291.4 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
+GATE_UP_M16_TRAFFIC_BYTES = 25748800
 
 
 def algorithmic_bytes(m: int, k: int, n: int) -> int:
