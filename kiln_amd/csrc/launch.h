@@ -50,7 +50,7 @@ struct DecodeArgs {
     int lora_producers = 0;        // = lora_slices, <= 16
     int lora_steps_per_slice = 0;  // 32-value steps of K per producer
     const void *lora_a = nullptr;  // bf16 [r_total, K]
-    unsigned *lora_flags = nullptr;  // 17 words, zero between launches
+    unsigned *lora_flags = nullptr;  // 64 KiB (16 replicas of flags and counts, 4 KiB apart), zero between launches
     int lora_adapters = 0;         // 1...4
     int lora_ends[4] = {};         // exclusive end column of adapter i (r_total past the last adapter)
     float lora_scales[4] = {};     // its scale (0 past the last)
@@ -87,6 +87,7 @@ hipError_t launch_decode(const DecodeArgs &args, hipStream_t stream);
 bool decode_gmp_ok(const DecodeArgs &a);                        // does the plan fit the private-staging instance?
 bool decode_gmp_fold_ok(const DecodeArgs &a);                   // ... with the LoRA projection folded into the launch?
 hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream);
+hipError_t launch_decode_gmp_lora(const DecodeArgs &a, hipStream_t stream);  // its instances with the low-rank term (checked plan)
 
 // One launch of the mid-M kernel: runs of up to 64 rows (grid z) against the whole weight.
 struct MidArgs {

@@ -90,14 +90,19 @@ __device__ __forceinline__ void lora_add_from_lds(f32x4 &v, const LoraTail &lo, 
 // writes its slice of T with device-scope stores, waits until they are acknowledged and raises
 // its flag; the blocks that add the term look at the flags once, through one wavefront, before
 // the barrier that precedes their tile sums, and read T with ordinary loads behind it (no cache
-// on their die has seen those lines since the launch began).  The flag words and the reader count
-// behind them live in workspace that is all zero between launches: every adding block counts
-// itself after its look, and the last one to do so zeroes the words.  producers == 0: T comes
-// from a launch of its own.
+// on their die has seen those lines since the launch began).  The flag words and the reader counts
+// live in workspace that is all zero between launches: every adding block counts itself after
+// its look, and the last one to do so zeroes the words.  Hundreds of blocks looking at one
+// address, or counting on one, are served one after the other (measured: 231 single polls of one
+// 64-byte line, every flag already up, took up to 4 us, and as long again for their 231 atomic
+// adds on one counter): the flags therefore exist kLoraFoldReplicas times, 4 KiB apart, block b
+// looks at and counts on replica b % kLoraFoldReplicas, and whoever completes a replica's count
+// counts once more on a top word.  producers == 0: T comes from a launch of its own.
 struct LoraFold {
     const uint16_t *a_cat;   // bf16 [r_total, K]: the adapters' A matrices stacked along rows
     uint16_t *t;             // where the producers write T: [producers][t_rows][rp] bf16
-    unsigned *flags;         // kLoraFoldFlagWords words: one per producer, the reader count last
+    unsigned *flags;         // kLoraFoldReplicas x kLoraFoldReplicaWords words: per replica one flag per producer,
+                             // then the replica's reader count; the top count behind that in replica 0
     int producers;           // K slices of the projection
     int steps_per_slice;     // 32-value steps of K per slice
     int consumers;           // blocks that add the term
@@ -109,7 +114,11 @@ struct LoraFold {
 constexpr int kLoraFoldMaxProducers = 16;
 constexpr int kLoraFoldMaxAdapters = 4;
 constexpr int kLoraFoldStepsPerWave = 8;   // 32-value steps of K one producer wavefront takes, at most
-constexpr int kLoraFoldFlagWords = kLoraFoldMaxProducers + 1;
+constexpr int kLoraFoldReplicas = 16;
+constexpr int kLoraFoldReplicaWords = 1024;                  // 4 KiB from one replica to the next
+constexpr int kLoraFoldCountWord = kLoraFoldMaxProducers;    // a replica's reader count
+constexpr int kLoraFoldTopWord = kLoraFoldMaxProducers + 1;  // in replica 0: completed replicas
+constexpr size_t kLoraFoldFlagBytes = (size_t)kLoraFoldReplicas * kLoraFoldReplicaWords * sizeof(unsigned);
 constexpr int kLoraFoldSpinLimit = 1 << 20;
 
 // One producer block: slice `slice` of T = scale(j) * x * a_cat^T for up to 16 rows of x (bf16 [M, K]),
@@ -178,30 +187,44 @@ __device__ __forceinline__ void lora_project_slice(const uint16_t *__restrict__ 
     }
     asm volatile("s_waitcnt vmcnt(0)" : : : "memory");  // this wavefront's part of T has reached memory
     __syncthreads();
-    if (wave == 0 && lane == 0)
-        __hip_atomic_store(fold.flags + slice, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0 && lane < kLoraFoldReplicas)
+        __hip_atomic_store(fold.flags + lane * kLoraFoldReplicaWords + slice, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// A block that adds the term, one wavefront of it, before the block's barrier: wait until every
+// A block that adds the term (the `consumer`-th of them), one wavefront of it: wait until every
 // producer has raised its flag.  The bound is never reached in a working launch.
-__device__ __forceinline__ void lora_fold_wait(const LoraFold &fold, int lane) {
-    for (int spins = 0; spins < kLoraFoldSpinLimit; ++spins) {
+__device__ __forceinline__ int lora_fold_wait(const LoraFold &fold, int consumer, int lane) {
+    const unsigned *mine = fold.flags + (consumer % kLoraFoldReplicas) * kLoraFoldReplicaWords;
+    int spins = 0;
+    for (; spins < kLoraFoldSpinLimit; ++spins) {
         unsigned f = 1u;
-        if (lane < fold.producers) f = __hip_atomic_load(fold.flags + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane < fold.producers) f = __hip_atomic_load(mine + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__builtin_amdgcn_ballot_w64(f == 0u) == 0) break;
         __builtin_amdgcn_s_sleep(4);
     }
+    return spins;  // polls that came back without every flag
 }
 
-// The same wavefront, after the barrier: count this block; the last block to do so has seen
-// every other block past its look at the flags and zeroes flags and count for the next launch.
-__device__ __forceinline__ void lora_fold_done(const LoraFold &fold, int lane) {
+// The same wavefront, after its look: count this block on its replica; the block that completes a
+// replica counts on the top word, and the one that completes that has seen every other block
+// past its look at the flags and zeroes flags and counts for the next launch.
+__device__ __forceinline__ void lora_fold_done(const LoraFold &fold, int consumer, int lane) {
+    const int replica = consumer % kLoraFoldReplicas;
+    const unsigned quota = (unsigned)(fold.consumers - replica + kLoraFoldReplicas - 1) / kLoraFoldReplicas;
+    const unsigned replicas = (unsigned)min(fold.consumers, kLoraFoldReplicas);
     unsigned before = 0;
     if (lane == 0)
-        before = __hip_atomic_fetch_add(fold.flags + kLoraFoldMaxProducers, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        before = __hip_atomic_fetch_add(fold.flags + replica * kLoraFoldReplicaWords + kLoraFoldCountWord, 1u,
+                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     before = (unsigned)__builtin_amdgcn_readfirstlane((int)before);
-    if (before == (unsigned)fold.consumers - 1u && lane < kLoraFoldFlagWords)
-        __hip_atomic_store(fold.flags + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (before != quota - 1u) return;
+    if (lane == 0)
+        before = __hip_atomic_fetch_add(fold.flags + kLoraFoldTopWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = (unsigned)__builtin_amdgcn_readfirstlane((int)before);
+    if (before != replicas - 1u) return;
+    if (lane <= kLoraFoldTopWord)
+        for (int r = 0; r < kLoraFoldReplicas; ++r)
+            __hip_atomic_store(fold.flags + r * kLoraFoldReplicaWords + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 inline LoraTail lora_tail(const DecodeArgs &a) {

@@ -19,8 +19,9 @@ constexpr size_t kCounterBytes = 64 * 1024;   // arrival counters at the start o
 // wavefront that adds a tile's parts writes zeros back), and a written word is never zero.
 constexpr size_t kFlaggedBytes = 4 * 1024 * 1024;
 constexpr size_t kZeroedBytes = kCounterBytes + kFlaggedBytes;
-// the last words of that region: producer flags and reader count of a LoRA projection folded into its GEMM launch
-constexpr size_t kFoldFlagBytes = 4096;
+// the end of that region: producer flags and reader counts of a LoRA projection folded into its GEMM
+// launch (16 replicas, 4 KiB apart: lora_tail.h)
+constexpr size_t kFoldFlagBytes = 16 * 4096;
 constexpr size_t kFoldFlagOffset = kCounterBytes + kFlaggedBytes - kFoldFlagBytes;
 
 struct DeviceInfo {
@@ -743,7 +744,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     int rp = 0, lora_slices = 1;
     // Up to 16 rows on the private-staging kernel: the projection rides in the GEMM launch (extra
     // blocks at the front of its grid) instead of running as a launch of its own.
-    DecodeArgs fold_probe;
+    DecodeArgs fold_probe{};
     bool fold = false;
     int fold_steps = 0;
     if (lora && g_tune.lora_fold != 0 && gp.launches == 1 && gp.dl[0].plan.gmp && gp.dl[0].M == prob_m) {
@@ -753,6 +754,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         kz = (steps + fold_steps - 1) / fold_steps;
         fold_probe.M = prob_m;
         fold_probe.K = prob_k;
+        fold_probe.KS = gp.dl[0].plan.KS;
         fold_probe.GS = gp.dl[0].plan.GS;
         fold_probe.waves = gp.dl[0].plan.waves;
         fold_probe.gm_tiles = gp.dl[0].plan.gm_tiles;

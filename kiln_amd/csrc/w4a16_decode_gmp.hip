@@ -32,8 +32,20 @@ constexpr int kGmpSlotBytes = 16 * 256;  // one group of A: 16 rows x 128 bf16
 #ifndef KILN_GMP_HEAD
 #define KILN_GMP_HEAD 3
 #endif
+// This file is compiled twice: as it is for calls without adapters, and with -DKILN_GMP_LORA=1 for
+// calls with them (launch_decode_gmp_lora only).  What the low-rank term adds -- one wavefront more,
+// its arguments, the signalling between the wavefronts -- then costs calls without adapters
+// nothing: as one kernel with run-time branches it cost them 0.1...0.2 us per launch.
+#ifndef KILN_GMP_LORA
+#define KILN_GMP_LORA 0
+#endif
+constexpr bool kGmpLora = KILN_GMP_LORA != 0;
+
 // Probe builds only (-DKILN_GMP_TIMELINE): wall-clock stamps (100 MHz) per wavefront.
 #ifdef KILN_GMP_TIMELINE
+#if KILN_GMP_LORA
+#define g_gmp_tl g_gmp_tl_lora
+#endif
 __device__ long long *g_gmp_tl;
 #define KILN_GMP_TL(i, v) tl_[i] = (v)
 #define KILN_GMP_NOW() ((long long)__builtin_amdgcn_s_memrealtime())
@@ -101,25 +113,30 @@ constexpr int gmp_slots(int gpw) { return gpw < 2 ? gpw : 2; }
 constexpr int kGmpFlaggedSlices = kDecodeFlaggedMaxSlices;  // most K slices the counter-free exchange takes
 constexpr int kGmpSpinLimit = 1 << 20;  // polls of the other slices' parts before the adding wavefront gives up
 
-// `units` 16-byte units from global memory to LDS by one wavefront, eight requests per lane in flight.
-__device__ __forceinline__ void copy_to_lds(unsigned char *dst, const uint16_t *src, int units, int lane) {
-    const u32x4 *s = reinterpret_cast<const u32x4 *>(src);
-    u32x4 *d = reinterpret_cast<u32x4 *>(dst);
-    for (int base = 0; base < units; base += 8 * 64) {
-        u32x4 r[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int u = base + 64 * i + lane;
-            r[i] = u32x4{0u, 0u, 0u, 0u};
-            if (u < units) r[i] = s[u];
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const int u = base + 64 * i + lane;
-            if (u < units) d[u] = r[i];
-        }
+// `units` 16-byte units from global memory (src: the same for the whole wavefront) to LDS at lds_addr
+// by one wavefront, 1 KiB per LDS-direct load, all of them in flight at once; done when the
+// wavefront's vector loads have landed.  The last load re-reads the last unit in its spare lanes:
+// up to 1 KiB - 16 bytes behind the destination are overwritten.
+__device__ __forceinline__ void copy_to_lds(unsigned lds_addr, const uint16_t *src, int units, int lane) {
+    for (int base = 0; base < units; base += 64)
+        load_to_lds_b128(src, (uint32_t)min(base + lane, units - 1) * 16u, lds_addr + (unsigned)base * 16u);
+}
+
+// One word of LDS as a signal from the adapter wavefront to the wavefronts that add the low-rank
+// term: LDS serves its requests in order, so whoever reads the word set reads the operands that
+// were written before it.  The wait is bounded like every other wait here.
+__device__ __forceinline__ void lds_signal_store(unsigned lds_addr, uint32_t value) {
+    asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : : "v"(lds_addr), "v"(value) : "memory");
+}
+__device__ __forceinline__ void lds_signal_wait(unsigned lds_addr, int at_least) {
+    for (int spins = 0; spins < kGmpSpinLimit; ++spins) {
+        uint32_t seen;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=v"(seen) : "v"(lds_addr) : "memory");
+        if (__builtin_amdgcn_readfirstlane((int)seen) >= at_least) break;
+        __builtin_amdgcn_s_sleep(1);
     }
 }
+constexpr uint32_t kGmpLooked = 1, kGmpOperandsReady = 2;  // values of the signal word
 
 // The kernel's last argument and where it sits among the arguments: the kernel reads it late, through
 // the argument segment's address (see there), so its place is spelled out as a struct with the
@@ -141,15 +158,47 @@ struct GmpKernelArgs {
 constexpr int kGmpLoraArgsOffset = (int)offsetof(GmpKernelArgs, la);
 static_assert(sizeof(GmpLoraArgs) % 4 == 0, "read word by word");
 
+// What only the end of the kernel needs -- where the result and the partial tiles go, how a tile is
+// stored -- waits in vector registers, of which the kernel has plenty, while the main loop uses
+// every scalar register there is for its addresses.
+struct GmpTailArgs {
+    uint16_t *C;
+    float *partial;
+    int *counters;
+    int swiglu, flagged;
+};
+struct GmpParkedTail {
+    uint32_t w[8];
+};
+__device__ __forceinline__ GmpParkedTail gmp_park(const GmpTailArgs &t) {
+    struct Words {
+        uint32_t w[8];
+    } in = __builtin_bit_cast(Words, t);
+    GmpParkedTail p;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(p.w[i]) : "s"(in.w[i]));
+    return p;
+}
+__device__ __forceinline__ GmpTailArgs gmp_unpark(const GmpParkedTail &p) {
+    struct Words {
+        uint32_t w[8];
+    } out;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) out.w[i] = (uint32_t)__builtin_amdgcn_readfirstlane((int)p.w[i]);
+    return __builtin_bit_cast(GmpTailArgs, out);
+}
+static_assert(sizeof(GmpTailArgs) == 32, "eight words");
+
 // T tiles per block, GPW groups per wavefront (the first `full_waves` wavefronts; the others one
 // fewer), AQ = LDS-direct loads per group of A: 4 (16 rows), 2 (M <= 8) or 1 (M <= 4: rows 0...3
 // only; the other rows of the product are computed from whatever LDS holds and never stored).
-template <int T, int GPW, int AQ>
+template <int T, int GPW, int AQ, bool LORA>
 __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     const uint16_t *__restrict__ A, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
-    uint16_t *__restrict__ C, float *partial, int *counters, int M, int N, int K, int Gs, int KS, int GS,
-    int full_waves, int slot_bytes, int col_shift, int producers, int adapter, int col_blocks, int nw_all,
-    int swiglu, int flagged, GmpLoraArgs la) {
+    uint16_t *__restrict__ C_arg, float *partial_arg, int *counters_arg, int M, int N, int K, int Gs, int KS, int GS,
+    int full_waves, int slot_bytes, int col_shift, int producers_arg, int adapter_arg, int col_blocks, int nw_all,
+    int swiglu_arg, int flagged_arg, GmpLoraArgs la) {
+    const int producers = LORA ? producers_arg : 0, adapter = LORA ? adapter_arg : 0;
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
 #ifdef KILN_GMP_TIMELINE
     long long tl_[8] = {};
@@ -160,6 +209,8 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     // round trip (0.2 us) between the launch and the first weight request.
     asm volatile("" : : "s"(A), "s"(B), "s"(S), "s"(M), "s"(N), "s"(K), "s"(Gs), "s"(KS), "s"(GS), "s"(full_waves),
                  "s"(slot_bytes), "s"(col_shift), "s"(producers), "s"(adapter), "s"(col_blocks), "s"(nw_all));
+    [[maybe_unused]] GmpParkedTail parked_tail;
+    if constexpr (LORA) parked_tail = gmp_park(GmpTailArgs{C_arg, partial_arg, counters_arg, swiglu_arg, flagged_arg});
     constexpr int NS = gmp_slots(GPW);
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -170,26 +221,33 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     const bool adapter_wave = wave == nw;  // never true without adapters
     const int G = K / kGroupK;
     const int NT = N / kTileN;
-    const int ks = blockIdx.y;
-    // With adapters whose projection is folded into this launch, the first `producers` blocks of
-    // the first slice compute it (the same block indices of the other slices have nothing to do).
-    if (__builtin_expect((int)blockIdx.x < producers, 0)) {
-        if (ks == 0) lora_project_slice(A, la.fold, la.lo, M, K, blockIdx.x, lds, wave, lane, nw_all);
+    // Calls without a folded projection: grid (column blocks, K slices).  With one, a single row
+    // of blocks: the `producers` blocks that compute it first, then the slices one after the other
+    // (a second grid dimension would launch the producers' indices once per slice, and the idle
+    // ones delay as many working blocks of the last slice by a round).
+    int ks = blockIdx.y, bx = blockIdx.x;
+    if (__builtin_expect(producers > 0, 0)) {
+        if (bx < producers) {
+            lora_project_slice(A, la.fold, la.lo, M, K, bx, lds, wave, lane, nw_all);
 #ifdef KILN_GMP_TIMELINE
-        if (ks == 0 && lane == 0 && g_gmp_tl) {
-            long long *o = g_gmp_tl + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 8;
-            o[0] = tl_[0];
-            o[6] = KILN_GMP_NOW();
-            o[7] = 100;
-        }
+            if (lane == 0 && g_gmp_tl) {
+                long long *o = g_gmp_tl + ((size_t)blockIdx.x * 16 + wave) * 8;
+                o[0] = tl_[0];
+                o[6] = KILN_GMP_NOW();
+                o[7] = 100;
+            }
 #endif
-        return;
+            return;
+        }
+        bx -= producers;  // at most four slices with a folded projection (decode_gmp_fold_ok)
+        ks = (bx >= col_blocks ? 1 : 0) + (bx >= 2 * col_blocks ? 1 : 0) + (bx >= 3 * col_blocks ? 1 : 0);
+        bx -= ks * col_blocks;
     }
     // Blocks go to the eight dies round-robin by linear index.  With the counter-free exchange the
     // column block is shifted by col_shift per slice, so that the slices of a tile sit on different
     // dies: a device-scope store and the device-scope load that polls it are slow when they meet
     // in one die's L2 (measured: 2...3 us per poll instead of 0.5).
-    const int col_block = (int)((blockIdx.x - producers + ks * col_shift) % col_blocks);
+    const int col_block = (bx + ks * col_shift) % col_blocks;
     const int tf = col_block * T;  // first tile of the block; tiles from NT on do not exist
     const bool full = wave < full_waves;
     const int g_first = full ? wave * GPW : full_waves * GPW + (wave - full_waves) * (GPW - 1);
@@ -314,29 +372,70 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     // finishes it.  Its operands come from LDS behind the main wavefronts' slots: the adapter
     // wavefront copies the rows of B_cat that belong to the block's tiles at once, and T -- all of
     // it, [slices][M][rp] -- as soon as it exists: with the projection folded into this launch, when
-    // every producer's flag is up.  All of it normally lands before the slowest main wavefront
-    // reaches the barrier, so the term costs a few LDS reads and products per tile.
+    // every producer's flag is up.  It does not hold up the block's barrier for that: the tiles are
+    // summed (and exchanged between K slices) while T is on its way, and a word of LDS tells the
+    // summing wavefronts when the operands are there.
     unsigned char *lora_b_lds = lds + nw * slot_bytes;
-    unsigned char *lora_t_lds = lora_b_lds + ((T * kTileN * lo.r_total * 2 + 15) & ~15);
+    const int lora_b_bytes = (T * kTileN * lo.r_total * 2 + 15) & ~15;
+    unsigned char *lora_t_lds = lora_b_lds + lora_b_bytes;
+    // (both evaluated where they are used: no scalar register held across the barrier)
+    auto lora_t_units = [&] { return lo.slices * lo.t_rows * lo.rp / 8; };
+    // the signal word sits behind T and the KiB that the copy of T may overwrite
+    auto lora_ready_addr = [&] { return (unsigned)(size_t)(lds_ptr_t)lora_t_lds + (unsigned)lora_t_units() * 16u + 1024u; };
     const bool adds_term = adapter != 0 && ks == KS - 1;
+    // Once the block has looked at the producers' flags it counts itself (the last block to do so
+    // zeroes them for the next launch): two atomics in a row across the chip, which the last main
+    // wavefront takes on where it has no tile to sum, so that they do not end the launch.
+    auto counting_wave_exists = [&] { return nw - 1 >= min(T, NT - tf); };
     if (__builtin_expect(adapter_wave && adds_term, 0)) {
+        lds_signal_store(lora_ready_addr(), 0u);
         const int live_tiles = min(T, NT - tf);
-        copy_to_lds(lora_b_lds, lo.b + (size_t)tf * kTileN * lo.r_total, live_tiles * kTileN * lo.r_total / 8, lane);
-        if (producers > 0) {
-            KILN_GMP_TL(3, KILN_GMP_NOW());
-            lora_fold_wait(fold, lane);
-            KILN_GMP_TL(4, KILN_GMP_NOW());
-        }
-        copy_to_lds(lora_t_lds, lo.t, lo.slices * lo.t_rows * lo.rp / 8, lane);
+        copy_to_lds((unsigned)(size_t)(lds_ptr_t)lora_b_lds, lo.b + (size_t)tf * kTileN * lo.r_total,
+                    live_tiles * kTileN * lo.r_total / 8, lane);
     }
-    __syncthreads();
+    __syncthreads();  // every wavefront's partial tiles are in LDS
     KILN_GMP_TL(2, KILN_GMP_NOW());
     if (__builtin_expect(adapter_wave, 0)) {
-        // count this block; the last one zeroes the producers' flags for the next launch
-        if (adds_term && producers > 0) lora_fold_done(fold, lane);
+        // The other wavefronts sum and exchange their tiles meanwhile; this one waits for T (with the
+        // projection folded into the launch: for every producer's flag), copies it behind the rows
+        // of B -- loads land in issue order, so what the copy of B overwrote behind its end is
+        // overwritten again -- and signals.
+        if (adds_term) {
+            if (fold.producers > 0) {
+                KILN_GMP_TL(3, KILN_GMP_NOW());
+                [[maybe_unused]] const int polls = lora_fold_wait(fold, tf / T, lane);
+                KILN_GMP_TL(4, KILN_GMP_NOW());
+                KILN_GMP_TL(5, (long long)polls + 1);
+                lds_signal_store(lora_ready_addr(), kGmpLooked);
+            }
+            copy_to_lds((unsigned)(size_t)(lds_ptr_t)lora_t_lds, lo.t, lora_t_units(), lane);
+            wait_vector_loads<0>();
+            lds_signal_store(lora_ready_addr(), kGmpOperandsReady);
+            if (fold.producers > 0 && !counting_wave_exists()) lora_fold_done(fold, tf / T, lane);
+        }
+#ifdef KILN_GMP_TIMELINE
+        if (lane == 0 && g_gmp_tl) {
+            long long *o = g_gmp_tl + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 8;
+            for (int i = 0; i < 6; ++i) o[i] = tl_[i];
+            o[6] = KILN_GMP_NOW();
+            o[7] = 200;
+        }
+#endif
         return;
     }
 
+    if (__builtin_expect(adds_term && fold.producers > 0 && wave == nw - 1 && counting_wave_exists(), 0)) {
+        lds_signal_wait(lora_ready_addr(), kGmpLooked);
+        lora_fold_done(fold, tf / T, lane);  // tf / T: the column block
+        return;
+    }
+
+    GmpTailArgs tail{C_arg, partial_arg, counters_arg, swiglu_arg, flagged_arg};
+    if constexpr (LORA) tail = gmp_unpark(parked_tail);
+    uint16_t *const C = tail.C;
+    float *const partial = tail.partial;
+    int *const counters = tail.counters;
+    const int swiglu = tail.swiglu, flagged = tail.flagged;
     const int q4 = lane >> 4, c = lane & 15;
     const int tiles = min(T, NT - tf);
     for (int ti = wave; ti < tiles; ti += nw) {
@@ -421,12 +520,15 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             }
             KILN_GMP_TL(4, KILN_GMP_NOW());
         }
-        if (adapter) lora_add_from_lds(sum, lo, lora_t_lds, lora_b_lds, ti, M, lane);
+        if (adapter) {
+            lds_signal_wait(lora_ready_addr(), kGmpOperandsReady);  // the term's operands are in LDS
+            lora_add_from_lds(sum, lo, lora_t_lds, lora_b_lds, ti, M, lane);
+        }
         store_tile_rows(C, N, M, 4 * q4, tt, c, sum, swiglu != 0);
     }
 #ifdef KILN_GMP_TIMELINE
     tl_[6] = KILN_GMP_NOW();
-    tl_[7] = 1ll + blockIdx.y;
+    tl_[7] = 1ll + ks;
     if (lane == 0 && g_gmp_tl) {
         long long *o = g_gmp_tl + (((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + wave) * 8;
         for (int i = 0; i < 8; ++i) o[i] = tl_[i];
@@ -440,7 +542,8 @@ size_t gmp_adapter_lds_bytes(const DecodeArgs &a) {
     if (a.r_total <= 0) return 0;
     const size_t rp = (size_t)(a.r_total + 15) / 16 * 16;
     const size_t b_bytes = ((size_t)a.gm_tiles * kTileN * a.r_total * 2 + 15) & ~(size_t)15;
-    return b_bytes + (size_t)a.lora_slices * a.lora_rows * rp * 2;
+    // + the KiB that the LDS-direct copy of T may overwrite behind it, + the signal word
+    return b_bytes + (size_t)a.lora_slices * a.lora_rows * rp * 2 + 1024 + 16;
 }
 
 int gmp_slot_bytes(int gpw, int tiles) {
@@ -450,7 +553,7 @@ int gmp_slot_bytes(int gpw, int tiles) {
 
 template <int T, int GPW, int AQ>
 hipError_t launch_gmp_tga(const DecodeArgs &a, hipStream_t stream) {
-    const hipError_t attr = allow_dynamic_lds<&w4a16_decode_gmp_kernel<T, GPW, AQ>>(decode_max_lds_bytes());
+    const hipError_t attr = allow_dynamic_lds<&w4a16_decode_gmp_kernel<T, GPW, AQ, kGmpLora>>(decode_max_lds_bytes());
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int full_waves = a.GS - a.waves * (GPW - 1);
@@ -469,12 +572,12 @@ hipError_t launch_gmp_tga(const DecodeArgs &a, hipStream_t stream) {
         fold.e0 = e[0], fold.e1 = e[1], fold.e2 = e[2], fold.e3 = e[3];
         fold.s0 = sc[0], fold.s1 = sc[1], fold.s2 = sc[2], fold.s3 = sc[3];
     }
-    const int grid_x = col_blocks + fold.producers;
+    const dim3 grid = fold.producers > 0 ? dim3(fold.producers + col_blocks * a.KS, 1) : dim3(col_blocks, a.KS);
     const int adapter = a.r_total > 0 ? 1 : 0;  // one wavefront more: it fetches the low-rank term's operands
     const size_t lds_bytes = (size_t)a.waves * slot + gmp_adapter_lds_bytes(a);
-    w4a16_decode_gmp_kernel<T, GPW, AQ><<<dim3(grid_x, a.KS), (a.waves + adapter) * 64, lds_bytes, stream>>>(
+    w4a16_decode_gmp_kernel<T, GPW, AQ, kGmpLora><<<grid, (a.waves + adapter) * 64, lds_bytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
-        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, slot, a.flagged ? exchange_column_shift(grid_x) : 0, fold.producers,
+        a.N, a.K, a.Gs, a.KS, a.GS, full_waves, slot, a.flagged ? exchange_column_shift(col_blocks) : 0, fold.producers,
         adapter, col_blocks, a.waves + adapter, a.swiglu ? 1 : 0, a.flagged ? 1 : 0, GmpLoraArgs{lora_tail(a), fold});
     return hipGetLastError();
 }
@@ -508,6 +611,20 @@ hipError_t launch_gmp_t(const DecodeArgs &a, int gpw, hipStream_t stream) {
 
 }  // namespace
 
+#if KILN_GMP_LORA
+// The instances with the low-rank term; the caller (launch_decode_gmp) has checked the plan.
+hipError_t launch_decode_gmp_lora(const DecodeArgs &a, hipStream_t stream) {
+    const int gpw = (a.GS + a.waves - 1) / a.waves;
+    switch (a.gm_tiles) {
+        case 1: return launch_gmp_t<1>(a, gpw, stream);
+        case 2: return launch_gmp_t<2>(a, gpw, stream);
+        case 3: return launch_gmp_t<3>(a, gpw, stream);
+        case 4: return launch_gmp_t<4>(a, gpw, stream);
+        case 5: return launch_gmp_t<5>(a, gpw, stream);
+        default: return launch_gmp_t<6>(a, gpw, stream);
+    }
+}
+#else
 // The private-staging group-major instance: M <= 16 rows, 1...6 whole tiles per block in equal K
 // slices of any length, wavefronts of ceil(GS / waves) groups (or one fewer) with at most 16
 // chunks each; a.waves <= 16 and <= GS.
@@ -537,6 +654,7 @@ bool decode_gmp_fold_ok(const DecodeArgs &a) {
     if (a.lora_steps_per_slice < 1 || (long)a.lora_producers * a.lora_steps_per_slice * 32 < a.K) return false;
     if (a.waves < jt || (a.lora_steps_per_slice + a.waves / jt - 1) / (a.waves / jt) > kLoraFoldStepsPerWave ||
         a.lora_rows != a.M || a.lora_adapters < 1 || a.lora_adapters > kLoraFoldMaxAdapters) return false;
+    if (a.KS > 4) return false;  // the kernel finds a block's slice in a one-row grid by three comparisons
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     return gmp_slot_bytes(gpw, a.gm_tiles) >= 1024;
 }
@@ -546,6 +664,7 @@ hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream) {
     if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
     if (a.flagged && a.KS > kGmpFlaggedSlices) return hipErrorInvalidValue;
     if (a.lora_producers > 0 && !decode_gmp_fold_ok(a)) return hipErrorInvalidValue;
+    if (a.r_total > 0) return launch_decode_gmp_lora(a, stream);
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.gm_tiles) {
         case 1: return launch_gmp_t<1>(a, gpw, stream);
@@ -557,10 +676,16 @@ hipError_t launch_decode_gmp(const DecodeArgs &a, hipStream_t stream) {
     }
 }
 
+#endif  // KILN_GMP_LORA
+
 }  // namespace kiln
 
 #ifdef KILN_GMP_TIMELINE
+#if KILN_GMP_LORA
+extern "C" int kiln_gmp_timeline_lora(long long *buf) {
+#else
 extern "C" int kiln_gmp_timeline(long long *buf) {
+#endif
     return (int)hipMemcpyToSymbol(HIP_SYMBOL(kiln::g_gmp_tl), &buf, sizeof(buf));
 }
 #endif

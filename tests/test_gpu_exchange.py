@@ -146,7 +146,8 @@ def _lora_call(L, xt, bt, st, la, lb, ranks, scales, m, k, n, ws=None):
     (9, 4096, 2560, (64,)),             # the largest rank
     (16, 2560, 2560, (8, 8, 8, 8)),     # four adapters
     (16, 2560, 2560, (8, 8, 8, 8, 8)),  # five: the projection runs as a launch of its own
-    (16, 2560, 8192, (16, 32)),         # 256 column blocks: no compute unit left for producers, a launch of its own
+    (16, 2560, 8192, (16, 32)),         # planned with wider blocks than the plain call's 256, which leave no unit for producers
+    (16, 2560, 8192, (8, 8, 8, 8, 8)),  # five adapters on that shape: planned for a fold that then cannot happen
     (1, 256, 256, (8,)),                # two groups of K, one producer
 ])
 def test_lora_projection_inside_the_gemm_launch(oracle, m, k, n, ranks):
