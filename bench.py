@@ -35,8 +35,8 @@ GROUP = 128
 LAYERS = 16
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
-# copy (x1.9989 and x1.0): 12291.4 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
-GATE_UP_M16_TRAFFIC_BYTES = 25748800
+# copy (x1.9989 and x1.0): 12278.6 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
+GATE_UP_M16_TRAFFIC_BYTES = 25722600
 
 
 def algorithmic_bytes(m: int, k: int, n: int) -> int:
@@ -397,7 +397,7 @@ def main() -> int:
                    "wall_ms_per_step": round(wall_step / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_M16_TRAFFIC_BYTES,
-                     "kernel": "w4a16_decode_gmp_kernel<5, 2, 4> (gate+up, M=16, K=2560, N=18432)",
+                     "kernel": "w4a16_decode_gmp_kernel<5, 2, 4, false> (gate+up, M=16, K=2560, N=18432)",
                      "us_per_launch": round(us_gu, 3), "algorithmic_bytes_per_launch": bytes_gu},
         "cpu_baseline": cpu_baseline,
         "extra": extra,
