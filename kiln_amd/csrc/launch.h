@@ -157,6 +157,7 @@ hipError_t launch_prefill(const PrefillArgs &args, hipStream_t stream);
 // lora_t = bf16 [*slices][M][r_total rounded up to 16] = per-adapter scale * (A * lora_a^T) in K slices,
 // padding columns zero.  few_rows: the small-M kernels will multiply it, in up to
 // prefill_lora_max_slices(M) slices; otherwise one slice.
-hipError_t launch_lora_project(const PrefillArgs &args, bool few_rows, hipStream_t stream, int *slices);
+hipError_t launch_lora_project(const PrefillArgs &args, bool few_rows, hipStream_t stream, int *slices,
+                               bool with_row_sums = false);  // many rows: also write the extension operand (args.aext)
 
 }  // namespace kiln

@@ -40,14 +40,17 @@ constexpr int kAStages = 4;
 // c[m][g] = -136 * sum_{k in group g} a[m][k], split into bf16 hi/mid/lo and
 // stored (group-major, [g][m]) as the 8-slot extension operand
 // [hi, hi, mid, mid, lo, lo, 0, 0].
-__global__ __launch_bounds__(256) void w4a16_prefill_rowsum_kernel(const uint16_t *__restrict__ A,
-                                                                 u32x4 *__restrict__ aext, int M, int K) {
-    const int G = K / kGroupK;
-    const int item = blockIdx.x * 16 + (threadIdx.x >> 4);  // (row, group), 16 lanes each
-    const int sub = threadIdx.x & 15;
-    if (item >= M * G) return;
-    const int row = item / G, g = item - row * G;
-    const u32x4 v = *reinterpret_cast<const u32x4 *>(A + (size_t)row * K + (size_t)g * kGroupK + sub * 8);
+__device__ __forceinline__ u32x4 extension_operand(float sum) {
+    const float c = -kCodeBias * sum;
+    const uint32_t hi = __builtin_bit_cast(uint32_t, c) & 0xFFFF0000u;
+    const float r1 = c - __builtin_bit_cast(float, hi);                     // exact
+    const uint32_t mid = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
+    const float r2 = r1 - __builtin_bit_cast(float, mid);                   // exact, <= 8 significant bits
+    const uint32_t lo = __builtin_bit_cast(uint32_t, r2) & 0xFFFF0000u;
+    return u32x4{(hi >> 16) | hi, (mid >> 16) | mid, (lo >> 16) | lo, 0u};
+}
+// the sum of 8 bf16 values in a 128-bit unit, in the order both kernels below use
+__device__ __forceinline__ float sum_bf16x8(u32x4 v) {
     const uint32_t wd[4] = {v.x, v.y, v.z, v.w};
     float sum = 0.f;
 #pragma unroll
@@ -55,22 +58,19 @@ __global__ __launch_bounds__(256) void w4a16_prefill_rowsum_kernel(const uint16_
         sum += __builtin_bit_cast(float, wd[i] << 16);
         sum += __builtin_bit_cast(float, wd[i] & 0xFFFF0000u);
     }
+    return sum;
+}
+__global__ __launch_bounds__(256) void w4a16_prefill_rowsum_kernel(const uint16_t *__restrict__ A,
+                                                                 u32x4 *__restrict__ aext, int M, int K) {
+    const int G = K / kGroupK;
+    const int item = blockIdx.x * 16 + (threadIdx.x >> 4);  // (row, group), 16 lanes each
+    const int sub = threadIdx.x & 15;
+    if (item >= M * G) return;
+    const int row = item / G, g = item - row * G;
+    float sum = sum_bf16x8(*reinterpret_cast<const u32x4 *>(A + (size_t)row * K + (size_t)g * kGroupK + sub * 8));
 #pragma unroll
     for (int off = 8; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 16);
-    if (sub == 0) {
-        const float c = -kCodeBias * sum;
-        const uint32_t hi = __builtin_bit_cast(uint32_t, c) & 0xFFFF0000u;
-        const float r1 = c - __builtin_bit_cast(float, hi);                     // exact
-        const uint32_t mid = __builtin_bit_cast(uint32_t, r1) & 0xFFFF0000u;
-        const float r2 = r1 - __builtin_bit_cast(float, mid);                   // exact, <= 8 significant bits
-        const uint32_t lo = __builtin_bit_cast(uint32_t, r2) & 0xFFFF0000u;
-        u32x4 o;
-        o.x = (hi >> 16) | hi;
-        o.y = (mid >> 16) | mid;
-        o.z = (lo >> 16) | lo;
-        o.w = 0u;
-        aext[(size_t)g * M + row] = o;  // group-major: the 32 rows of a half-wavefront are contiguous
-    }
+    if (sub == 0) aext[(size_t)g * M + row] = extension_operand(sum);  // group-major: the 32 rows of a half-wavefront are contiguous
 }
 
 // T[m][j] = bf16(scale(j) * sum_k x[m][k] * a_cat[j][k]) for the stacked LoRA A matrices (rows j
@@ -108,7 +108,7 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
                                                                 const uint16_t *__restrict__ a_cat,
                                                                 uint16_t *__restrict__ T, int M, int K, int r_total,
                                                                 int RP, int steps_per_slice, LoraScales ls,
-                                                                float *partial, int *counters) {
+                                                                float *partial, int *counters, u32x4 *aext) {
     extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
     constexpr int XL = RB * 32 / 256;                // 128-bit loads per thread and piece: x ...
     constexpr int AL = kProjectMaxRank * 32 / 256;   // ... and a_cat (rows from r_total on are not read)
@@ -172,6 +172,22 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
                 *reinterpret_cast<u32x4 *>(a_lds + (pr + 8 * i) * kProjectRowBytes + pc * 16) = ar[b][i];
         __syncthreads();
         if (c0 + 2 * kPieceSteps < s1) request(buf, c0 + 2 * kPieceSteps);
+        if (aext) {
+            // The matrix-core kernel's extension operand (see w4a16_prefill_rowsum_kernel, whose launch
+            // this saves): the staged piece of x holds two whole groups of every row of the block --
+            // slices are whole groups, so each (row, group) is formed exactly once.  16 lanes per item,
+            // same order of additions as the kernel above.
+            const int sub = tid & 15;
+#pragma unroll
+            for (int base = 0; base < RB * 2; base += 16) {
+                const int it2 = base + (tid >> 4), row = it2 >> 1, half = it2 & 1;
+                float sum = sum_bf16x8(*reinterpret_cast<const u32x4 *>(x_lds + row * kProjectRowBytes + half * 256 + sub * 16));
+#pragma unroll
+                for (int off = 8; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 16);
+                if (sub == 0 && m0 + row < M && c0 + 4 * half < s1)
+                    aext[(size_t)(c0 / 4 + half) * M + m0 + row] = extension_operand(sum);
+            }
+        }
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
             const int item = wave + 4 * it;
@@ -1015,7 +1031,7 @@ int lora_project_slices(int m, int k) {
     return kz < 1 ? 1 : kz;
 }
 
-hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t stream, int *slices) {
+hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t stream, int *slices, bool with_row_sums) {
     if (a.r_total < 1 || a.r_total > kProjectMaxRank || a.n_adapters < 1 || a.n_adapters > 8 || !a.lora_a ||
         !a.lora_t || !a.ranks || !a.scales || a.M < 1 || a.K < kGroupK)
         return hipErrorInvalidValue;
@@ -1030,6 +1046,8 @@ hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t 
     }
     *slices = 1;
     const int steps = a.K / 32;
+    u32x4 *aext = with_row_sums && !few_rows ? (u32x4 *)a.aext : nullptr;
+    if (with_row_sums && !aext) return hipErrorInvalidValue;
     if (!few_rows) {
         // many rows: T whole.  K slices that meet in f32 behind T, as many as keep about 256 blocks busy.
         const int rb = lora_project_rows_per_block(a.M, a.K), row_tiles = (a.M + rb - 1) / rb;
@@ -1046,13 +1064,13 @@ hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t 
         if (rb == 16) {
             w4a16_lora_project_kernel<16><<<dim3(row_tiles, kz), 256, lds_bytes, stream>>>(
                 (const uint16_t *)a.A, (const uint16_t *)a.lora_a, (uint16_t *)a.lora_t, a.M, a.K, a.r_total, RP,
-                per_slice, ls, partial, a.counters);
+                per_slice, ls, partial, a.counters, aext);
         } else {
             const hipError_t attr = allow_dynamic_lds<&w4a16_lora_project_kernel<64>>(lds_bytes);
             if (attr != hipSuccess) return attr;
             w4a16_lora_project_kernel<64><<<dim3(row_tiles, kz), 256, lds_bytes, stream>>>(
                 (const uint16_t *)a.A, (const uint16_t *)a.lora_a, (uint16_t *)a.lora_t, a.M, a.K, a.r_total, RP,
-                per_slice, ls, partial, a.counters);
+                per_slice, ls, partial, a.counters, aext);
         }
         return hipGetLastError();
     }
@@ -1063,7 +1081,7 @@ hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t 
     const int lds_bytes = (16 + kProjectMaxRank) * kProjectRowBytes + kProjectMaxRank * (int)sizeof(float);
     w4a16_lora_project_kernel<16><<<dim3((a.M + 15) / 16, kz), 256, lds_bytes, stream>>>(
         (const uint16_t *)a.A, (const uint16_t *)a.lora_a, (uint16_t *)a.lora_t, a.M, a.K, a.r_total, RP, per_slice, ls,
-        nullptr, nullptr);
+        nullptr, nullptr, nullptr);
     return hipGetLastError();
 }
 
@@ -1080,7 +1098,9 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     const double flops = 2.0 * a.M * (double)a.N * a.K;
     const bool rs = a.bm == 64 && row_sum_bytes(max_groups) <= kMaxRowSumBytes && (flops <= 28e9 || a.N <= 4096);
     hipError_t err = hipSuccess;
-    if (!rs) {
+    // with adapters the projection's launch forms the row sums on its way over x
+    const bool sums_with_projection = !rs && a.r_total > 0;
+    if (!rs && !sums_with_projection) {
         const int items = a.M * G;
         w4a16_prefill_rowsum_kernel<<<(items + 15) / 16, 256, 0, stream>>>((const uint16_t *)a.A, (u32x4 *)a.aext,
                                                                           a.M, a.K);
@@ -1091,7 +1111,7 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     if (a.r_total > 0) {
         RP = (a.r_total + 15) / 16 * 16;
         int slices = 1;  // many rows: T is whole
-        err = launch_lora_project(a, false, stream, &slices);
+        err = launch_lora_project(a, false, stream, &slices, sums_with_projection);
         if (err != hipSuccess) return err;
         if (slices != 1) return hipErrorInvalidValue;
     }
