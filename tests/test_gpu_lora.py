@@ -197,6 +197,29 @@ def test_lora_argument_errors():
     assert tuple(y.shape) == (2, 256)
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (512, 2560, 18432),    # 64-row blocks on a work-bound launch: the row sums come from a pre-pass
+    (333, 2560, 18432),    # ... with a ragged last row tile
+    (1100, 9216, 8192),    # 128-row blocks; the projection takes 64 rows per block
+    (1030, 2560, 8192),    # 128-row blocks, 16 rows per projection block
+])
+def test_adapters_with_zero_b_equal_the_plain_call_bit_for_bit(m, k, n):
+    """With adapters the projection's launch also writes the matrix-core kernel's row-sum operand (a
+    launch of its own without them).  B = 0 makes the low-rank term vanish, so the two calls must
+    agree in every bit: same operand, same order of additions."""
+    gen = torch.Generator(device="cuda").manual_seed(m + k + n)
+    bt = torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device="cuda", generator=gen)
+    st = (torch.rand(k // 128, n, device="cuda", generator=gen) * 0.018 + 0.002).to(torch.float16)
+    x = (torch.randn(m, k, device="cuda", generator=gen) * 0.5).to(torch.bfloat16)
+    ranks, scales = (16, 32), (0.5, 1.0)
+    a_cat = (torch.randn(sum(ranks), k, device="cuda", generator=gen) * 0.02).to(torch.bfloat16)
+    b_cat = torch.zeros(n, sum(ranks), dtype=torch.bfloat16, device="cuda")
+    plain = marlin_gemm.marlin_w4a16_gemm(x, bt, st, 128)
+    with_adapters = marlin_gemm.marlin_w4a16_gemm_lora(x, bt, st, 128, a_cat, b_cat, ranks, scales)
+    torch.cuda.synchronize()
+    assert torch.equal(plain.view(torch.int16), with_adapters.view(torch.int16))
+
+
 @pytest.mark.parametrize("m,k,n,ranks", [(200, 9216, 256, (7,)), (16, 9216, 2560, (16, 32))])
 def test_lora_run_to_run_determinism(oracle, m, k, n, ranks):
     """The projection's K slices meet as f32 tiles in the workspace (many rows) and the GEMM's own
