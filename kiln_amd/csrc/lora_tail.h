@@ -88,9 +88,9 @@ __device__ __forceinline__ void lora_add_from_lds(f32x4 &v, const LoraTail &lo, 
 // The projection T computed inside the launch that adds it, by `producers` extra blocks at the
 // front of the grid (one K slice each) while the other blocks stream their weights.  A producer
 // writes its slice of T with device-scope stores, waits until they are acknowledged and raises
-// its flag; the blocks that add the term look at the flags once, through one wavefront, before
-// the barrier that precedes their tile sums, and read T with ordinary loads behind it (no cache
-// on their die has seen those lines since the launch began).  The flag words and the reader counts
+// its flag; the blocks that add the term look at the flags through one wavefront (while the
+// others sum their tiles) and read T with ordinary loads once the flags are up (no cache on
+// their die has seen those lines since the launch began).  The flag words and the reader counts
 // live in workspace that is all zero between launches: every adding block counts itself after
 // its look, and the last one to do so zeroes the words.  Hundreds of blocks looking at one
 // address, or counting on one, are served one after the other (measured: 231 single polls of one
