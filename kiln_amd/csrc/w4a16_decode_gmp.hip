@@ -137,6 +137,13 @@ __device__ __forceinline__ void lds_signal_wait(unsigned lds_addr, int at_least)
     }
 }
 constexpr uint32_t kGmpLooked = 1, kGmpOperandsReady = 2;  // values of the signal word
+// A count in LDS that wavefronts raise (after their own LDS writes, which LDS serves first) and
+// others wait for: a barrier that only holds up those who need what the others wrote.
+__device__ __forceinline__ void lds_count_arrival(unsigned lds_addr, int lane) {
+    if (lane == 0) asm volatile("ds_add_u32 %0, %1" : : "v"(lds_addr), "v"(1u) : "memory");
+}
+// Two words at the start of the adapter wavefront's part of LDS: the signal and the arrival count.
+constexpr unsigned kGmpSyncBytes = 16;
 
 // The kernel's last argument and where it sits among the arguments: the kernel reads it late, through
 // the argument segment's address (see there), so its place is spelled out as a struct with the
@@ -299,6 +306,7 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
         using Sch = GmpScheduleOf<T, NGR, AQ>;
         unrolled<0, (kGmpHead < U ? kGmpHead : U)>(request_chunk);
         request_a(0, 0);
+        if constexpr (LORA) __syncthreads();  // the adapter wavefront has zeroed the words the block meets on
         u32x4 af[4];
         f32x4 offset_term;
         unrolled<0, U>([&](auto jc) {
@@ -347,6 +355,11 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
         f32x4 *slots = reinterpret_cast<f32x4 *>(mine);
 #pragma unroll
         for (int ti = 0; ti < T; ++ti) slots[ti * 64 + lane] = y[ti];
+    } else if constexpr (LORA) {
+        const unsigned sync_addr = (unsigned)(size_t)(lds_ptr_t)(lds + nw * slot_bytes);
+        lds_signal_store(sync_addr, 0u);
+        lds_signal_store(sync_addr + 4, 0u);
+        __syncthreads();  // pairs with the one behind the main wavefronts' first requests
     }
 
     // What the low-rank term needs is read from the kernel arguments only now: as ordinary
@@ -372,35 +385,40 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     // finishes it.  Its operands come from LDS behind the main wavefronts' slots: the adapter
     // wavefront copies the rows of B_cat that belong to the block's tiles at once, and T -- all of
     // it, [slices][M][rp] -- as soon as it exists: with the projection folded into this launch, when
-    // every producer's flag is up.  It does not hold up the block's barrier for that: the tiles are
-    // summed (and exchanged between K slices) while T is on its way, and a word of LDS tells the
-    // summing wavefronts when the operands are there.
-    unsigned char *lora_b_lds = lds + nw * slot_bytes;
+    // every producer's flag is up.  It holds up nobody with that: the tiles are summed (and exchanged
+    // between K slices) while T is on its way, and a word of LDS tells the summing wavefronts when
+    // the operands are there.
+    unsigned char *lora_b_lds = lds + nw * slot_bytes + kGmpSyncBytes;
     const int lora_b_bytes = (T * kTileN * lo.r_total * 2 + 15) & ~15;
     unsigned char *lora_t_lds = lora_b_lds + lora_b_bytes;
-    // (both evaluated where they are used: no scalar register held across the barrier)
+    // (evaluated where they are used: no scalar register held meanwhile)
     auto lora_t_units = [&] { return lo.slices * lo.t_rows * lo.rp / 8; };
-    // the signal word sits behind T and the KiB that the copy of T may overwrite
-    auto lora_ready_addr = [&] { return (unsigned)(size_t)(lds_ptr_t)lora_t_lds + (unsigned)lora_t_units() * 16u + 1024u; };
+    auto lora_ready_addr = [&] { return (unsigned)(size_t)(lds_ptr_t)(lds + nw * slot_bytes); };  // the signal word
+    auto arrivals_addr = [&] { return lora_ready_addr() + 4u; };                                   // the arrival count
     const bool adds_term = adapter != 0 && ks == KS - 1;
     // Once the block has looked at the producers' flags it counts itself (the last block to do so
     // zeroes them for the next launch): two atomics in a row across the chip, which the last main
     // wavefront takes on where it has no tile to sum, so that they do not end the launch.
     auto counting_wave_exists = [&] { return nw - 1 >= min(T, NT - tf); };
-    if (__builtin_expect(adapter_wave && adds_term, 0)) {
-        lds_signal_store(lora_ready_addr(), 0u);
-        const int live_tiles = min(T, NT - tf);
-        copy_to_lds((unsigned)(size_t)(lds_ptr_t)lora_b_lds, lo.b + (size_t)tf * kTileN * lo.r_total,
-                    live_tiles * kTileN * lo.r_total / 8, lane);
+    // Without adapters the block meets at a barrier.  With them it must not: the adapter wavefront
+    // waits for the producers, and the main wavefronts of a fast block would wait with it.  There the
+    // main wavefronts count their arrival in LDS, only those that sum a tile wait for the count, and
+    // the adapter wavefront runs beside them from the first instruction on.
+    if constexpr (!LORA) {
+        __syncthreads();  // every wavefront's partial tiles are in LDS
+    } else if (!adapter_wave) {
+        lds_count_arrival(arrivals_addr(), lane);
     }
-    __syncthreads();  // every wavefront's partial tiles are in LDS
     KILN_GMP_TL(2, KILN_GMP_NOW());
     if (__builtin_expect(adapter_wave, 0)) {
-        // The other wavefronts sum and exchange their tiles meanwhile; this one waits for T (with the
-        // projection folded into the launch: for every producer's flag), copies it behind the rows
-        // of B -- loads land in issue order, so what the copy of B overwrote behind its end is
-        // overwritten again -- and signals.
+        // This one copies the block's rows of B, waits for T (with the projection folded into the
+        // launch: for every producer's flag), copies it behind the rows of B -- loads land in
+        // issue order, so what the copy of B overwrote behind its end is overwritten again -- and
+        // signals.
         if (adds_term) {
+            const int live_tiles = min(T, NT - tf);
+            copy_to_lds((unsigned)(size_t)(lds_ptr_t)lora_b_lds, lo.b + (size_t)tf * kTileN * lo.r_total,
+                        live_tiles * kTileN * lo.r_total / 8, lane);
             if (fold.producers > 0) {
                 KILN_GMP_TL(3, KILN_GMP_NOW());
                 [[maybe_unused]] const int polls = lora_fold_wait(fold, tf / T, lane);
@@ -438,6 +456,9 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
     const int swiglu = tail.swiglu, flagged = tail.flagged;
     const int q4 = lane >> 4, c = lane & 15;
     const int tiles = min(T, NT - tf);
+    if constexpr (LORA) {
+        if (wave < tiles) lds_signal_wait(arrivals_addr(), nw);  // every main wavefront's partial tiles are in LDS
+    }
     for (int ti = wave; ti < tiles; ti += nw) {
         const int tt = tf + ti;
         // (requesting all wavefronts' parts at once and adding them behind selects measured
@@ -542,8 +563,8 @@ size_t gmp_adapter_lds_bytes(const DecodeArgs &a) {
     if (a.r_total <= 0) return 0;
     const size_t rp = (size_t)(a.r_total + 15) / 16 * 16;
     const size_t b_bytes = ((size_t)a.gm_tiles * kTileN * a.r_total * 2 + 15) & ~(size_t)15;
-    // + the KiB that the LDS-direct copy of T may overwrite behind it, + the signal word
-    return b_bytes + (size_t)a.lora_slices * a.lora_rows * rp * 2 + 1024 + 16;
+    // + the KiB that the LDS-direct copy of T may overwrite behind it, + the words the block meets on
+    return kGmpSyncBytes + b_bytes + (size_t)a.lora_slices * a.lora_rows * rp * 2 + 1024;
 }
 
 int gmp_slot_bytes(int gpw, int tiles) {
@@ -614,6 +635,7 @@ hipError_t launch_gmp_t(const DecodeArgs &a, int gpw, hipStream_t stream) {
 #if KILN_GMP_LORA
 // The instances with the low-rank term; the caller (launch_decode_gmp) has checked the plan.
 hipError_t launch_decode_gmp_lora(const DecodeArgs &a, hipStream_t stream) {
+    if (a.r_total <= 0) return hipErrorInvalidValue;  // these instances count on the adapter wavefront
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.gm_tiles) {
         case 1: return launch_gmp_t<1>(a, gpw, stream);
