@@ -913,7 +913,8 @@ int prefill_grid(int m, int n, const PrefillPlan &p) {
 // is cut into as many K slices as still leave one block per compute unit and three groups
 // per slice, so the last round is as full as the others instead of leaving most of the chip
 // idle.
-static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm) {
+static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm, int sliced_units = 0) {
+    if (sliced_units <= 0) sliced_units = cus;  // (tile, K slice) units the sliced round may have
     PrefillPlan p;
     p.bn = bn;
     p.bm = bm;
@@ -926,7 +927,7 @@ static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm) 
         const int gsb = (G + ks - 1) / ks;
         if ((ks - 1) * gsb >= G) continue;  // would leave an empty slice
         const int dr = prefill_die_rows(m_blocks), dc = 8 / dr;
-        if (8 * (m_blocks / dr) * ((rest * ks + dc - 1) / dc) <= cus) p.ks = ks;
+        if (8 * (m_blocks / dr) * ((rest * ks + dc - 1) / dc) <= sliced_units) p.ks = ks;
     }
     return p;
 }
@@ -957,13 +958,23 @@ static float plan_cost(int m, int n, int k, int cus, const PrefillPlan &p) {
 // The 256-row shapes stay available through the overrides.
 PrefillPlan plan_prefill(int m, int n, int k, int cus, int force_bn, int force_bm) {
     int bm = m <= 768 ? 64 : 128;
+    int sliced_units = 0;
     if (bm == 128) {
         const int tiles = ((m + 127) / 128) * (n / 256);
-        if (2 * tiles > cus && tiles < cus) bm = 64;
+        if (2 * tiles > cus && tiles < cus) {
+            // Tiles for 50...100 % of the compute units.  Two 128-row blocks fit a unit: with every tile
+            // cut into as many K slices as fill those slots the chip is busier than with 64-row blocks,
+            // provided a slice stays long (measured on N = 2560: K = 9216 at M = 2048 / 2560 / 3072, three
+            // or two slices of 24 or 36 groups, 121 / 148 / 162 us against 124 / 159 / 168; K = 4096 at
+            // M = 3072 in two slices of 16 groups 90 against 84)
+            const int ks = 2 * cus / tiles;
+            if (ks >= 2 && k / kGroupK / ks >= 24) sliced_units = 2 * cus;
+            else bm = 64;
+        }
     }
     if (force_bm == 64 || force_bm == 128 || force_bm == 256) bm = force_bm;
     if (force_bn == 128 || force_bn == 256) return plan_for_shape(m, n, k, cus, force_bn, bm);
-    const PrefillPlan wide = plan_for_shape(m, n, k, cus, 256, bm);
+    const PrefillPlan wide = plan_for_shape(m, n, k, cus, 256, bm, bm == 128 ? sliced_units : 0);
     if (bm == 128) return wide;
     const PrefillPlan narrow = plan_for_shape(m, n, k, cus, 128, bm);
     if (bm == 64) return plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, wide) ? narrow : wide;
