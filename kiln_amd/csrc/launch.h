@@ -138,6 +138,8 @@ struct PrefillArgs {
     int cus = 256;                  // compute units of the device
     float *partial = nullptr;       // prefill_partial_bytes(M, N, KS) bytes
     int *counters = nullptr;        // one per 256 x 128 tile, zero on entry and on exit
+    unsigned *lora_words = nullptr; // 64 KiB that are zero between launches (see lora_tail.h): with them the LoRA
+                                    // projection may run inside the product's launch; null: always in front of it
 };
 
 size_t prefill_aext_bytes(int m, int k);

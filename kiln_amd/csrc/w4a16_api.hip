@@ -716,6 +716,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             pa.n_adapters = lora->n_adapters;
             pa.ranks = lora->ranks;
             pa.scales = lora->scales;
+            if (g_tune.lora_fold != 0) pa.lora_words = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
         }
         pa.swiglu = swiglu;
         pa.cus = cus;

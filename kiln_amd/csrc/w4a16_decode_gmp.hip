@@ -139,7 +139,7 @@ __device__ __forceinline__ void lds_signal_wait(unsigned lds_addr, int at_least)
 constexpr uint32_t kGmpLooked = 1, kGmpOperandsReady = 2;  // values of the signal word
 // A count in LDS that wavefronts raise (after their own LDS writes, which LDS serves first) and
 // others wait for: a barrier that only holds up those who need what the others wrote.
-__device__ __forceinline__ void lds_count_arrival(unsigned lds_addr, int lane) {
+[[maybe_unused]] __device__ __forceinline__ void lds_count_arrival(unsigned lds_addr, int lane) {
     if (lane == 0) asm volatile("ds_add_u32 %0, %1" : : "v"(lds_addr), "v"(1u) : "memory");
 }
 // Two words at the start of the adapter wavefront's part of LDS: the signal and the arrival count.

@@ -30,6 +30,7 @@
 
 #include "device_common.h"
 #include "launch.h"
+#include "lora_tail.h"
 
 namespace kiln {
 
@@ -103,13 +104,25 @@ constexpr int kProjectPieceK = 256;                          // values of K per 
 constexpr int kProjectRowBytes = kProjectPieceK * 2 + 16;    // padded LDS row
 constexpr int kProjectMaxRank = 64;
 
+// A 128-bit store that is written through to memory (device scope).  A store of more than 64 bits
+// reads the upper part of its data registers after it has issued; the compiler pads that for its
+// own stores, not for one inside inline asm: hence the s_nop.
+__device__ __forceinline__ void store_b128_through(void *ptr, u32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off sc1\n\ts_nop 1" : : "v"(ptr), "v"(v) : "memory");
+}
+
+// The work of one block (256 threads): row tile `row_tile` (RB rows), K slice `slice` of `KZ`.
+// `done` (optional): a word per row tile, raised when the tile's rows of T (and, with `aext`, of the
+// extension operand) are in memory -- for a caller that computes the projection inside another
+// kernel's launch instead of in front of it.  Both are then written through to memory: an ordinary
+// store is complete when this die's cache has it, which a reader on another die does not see
+// before the launch ends.
 template <int RB>  // rows per block: 16 or 64
-__global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t *__restrict__ X,
-                                                                const uint16_t *__restrict__ a_cat,
-                                                                uint16_t *__restrict__ T, int M, int K, int r_total,
-                                                                int RP, int steps_per_slice, LoraScales ls,
-                                                                float *partial, int *counters, u32x4 *aext) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+__device__ __forceinline__ void lora_project_block(unsigned char *lds, const uint16_t *__restrict__ X,
+                                                   const uint16_t *__restrict__ a_cat, uint16_t *__restrict__ T, int M,
+                                                   int K, int r_total, int RP, int steps_per_slice, const LoraScales &ls,
+                                                   float *partial, int *counters, u32x4 *aext, int row_tile, int slice,
+                                                   int KZ, unsigned *done) {
     constexpr int XL = RB * 32 / 256;                // 128-bit loads per thread and piece: x ...
     constexpr int AL = kProjectMaxRank * 32 / 256;   // ... and a_cat (rows from r_total on are not read)
     constexpr int IT = RB / 16;                      // tiles of T per wavefront, at most
@@ -118,9 +131,9 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
     unsigned char *x_lds = lds, *a_lds = lds + RB * kProjectRowBytes;
     float *sc_lds = reinterpret_cast<float *>(lds + (RB + kProjectMaxRank) * kProjectRowBytes);
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int m0 = blockIdx.x * RB;
+    const int m0 = row_tile * RB;
     const int steps = K / 32;                        // steps of 32 values of K
-    const int s0 = blockIdx.y * steps_per_slice, s1 = min(steps, s0 + steps_per_slice);
+    const int s0 = slice * steps_per_slice, s1 = min(steps, s0 + steps_per_slice);
     const int rows = min(RB, M - m0), row_tiles = (rows + 15) >> 4, JT = RP >> 4;
     const int items = row_tiles * JT;
 
@@ -184,8 +197,11 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
                 float sum = sum_bf16x8(*reinterpret_cast<const u32x4 *>(x_lds + row * kProjectRowBytes + half * 256 + sub * 16));
 #pragma unroll
                 for (int off = 8; off >= 1; off >>= 1) sum += __shfl_xor(sum, off, 16);
-                if (sub == 0 && m0 + row < M && c0 + 4 * half < s1)
-                    aext[(size_t)(c0 / 4 + half) * M + m0 + row] = extension_operand(sum);
+                if (sub == 0 && m0 + row < M && c0 + 4 * half < s1) {
+                    u32x4 *dst = aext + (size_t)(c0 / 4 + half) * M + m0 + row;
+                    if (done) store_b128_through(dst, extension_operand(sum));
+                    else *dst = extension_operand(sum);
+                }
             }
         }
 #pragma unroll
@@ -213,21 +229,20 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
     }
     __syncthreads();  // sc_lds (a slice may be empty: then no barrier above)
 
-    uint16_t *Tz = T + (size_t)blockIdx.y * M * RP;
-    if (partial && gridDim.y > 1) {
+    uint16_t *Tz = T + (size_t)slice * M * RP;
+    if (partial && KZ > 1) {
         // One T for all of K: the slices of a row tile meet in `partial` as f32 tiles (device-scope
         // accesses); the last block to arrive adds them in slice order, so the result does not
         // depend on arrival order, and leaves the counter at zero.
         __shared__ int s_last;
-        const int KZ = gridDim.y;
-        float *tile0 = partial + (size_t)blockIdx.x * KZ * (IT * 4) * 256 + lane;  // [slice][item][4][64]
+        float *tile0 = partial + (size_t)row_tile * KZ * (IT * 4) * 256 + lane;  // [slice][item][4][64]
 #pragma unroll
         for (int it = 0; it < IT; ++it) {
             const int item = wave + 4 * it;
             if (item < items)
 #pragma unroll
                 for (int i = 0; i < 4; ++i)
-                    __hip_atomic_store(tile0 + ((size_t)(blockIdx.y * (IT * 4) + item) * 4 + i) * 64, acc[it][i],
+                    __hip_atomic_store(tile0 + ((size_t)(slice * (IT * 4) + item) * 4 + i) * 64, acc[it][i],
                                        __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         // each wavefront waits until its own stores have been acknowledged (a barrier alone
@@ -235,7 +250,7 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
         __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
         __syncthreads();
         if (tid == 0)
-            s_last = __hip_atomic_fetch_add(counters + blockIdx.x, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KZ - 1;
+            s_last = __hip_atomic_fetch_add(counters + row_tile, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KZ - 1;
         __syncthreads();
         if (!s_last) return;
         // every read is requested before the first is used: device-scope reads are slow, and this
@@ -257,7 +272,7 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
 #pragma unroll
             for (int z = 1; z < ZMAX; ++z) acc[it] += part[it][z];
         }
-        if (tid == 0) __hip_atomic_store(counters + blockIdx.x, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (tid == 0) __hip_atomic_store(counters + row_tile, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         Tz = T;
     }
 #pragma unroll
@@ -270,9 +285,35 @@ __global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t 
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = m0 + rt * 16 + 4 * (lane >> 4) + i;
-            if (r < M) Tz[(size_t)r * RP + j] = f32_to_bf16_bits(acc[it][i] * sc);
+            const uint32_t mine = f32_to_bf16_bits(acc[it][i] * sc);
+            if (done) {  // two neighbouring columns per 32-bit device-scope store (even lanes)
+                const uint32_t next = (uint32_t)__shfl_xor((int)mine, 1, 64);
+                if ((lane & 1) == 0 && r < M)
+                    __hip_atomic_store(reinterpret_cast<uint32_t *>(Tz + (size_t)r * RP + j), mine | (next << 16),
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else if (r < M) {
+                Tz[(size_t)r * RP + j] = (uint16_t)mine;
+            }
         }
     }
+    if (done) {
+        // whoever gets here wrote the tile's rows of T, after every slice's stores (its own included)
+        // had been acknowledged: the extension operand of all slices is in memory too
+        __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+        __syncthreads();
+        if (tid == 0) __hip_atomic_store(done + row_tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+template <int RB>
+__global__ __launch_bounds__(256) void w4a16_lora_project_kernel(const uint16_t *__restrict__ X,
+                                                                const uint16_t *__restrict__ a_cat,
+                                                                uint16_t *__restrict__ T, int M, int K, int r_total,
+                                                                int RP, int steps_per_slice, LoraScales ls,
+                                                                float *partial, int *counters, u32x4 *aext) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
+    lora_project_block<RB>(lds, X, a_cat, T, M, K, r_total, RP, steps_per_slice, ls, partial, counters, aext,
+                           blockIdx.x, blockIdx.y, gridDim.y, nullptr);
 }
 
 typedef __attribute__((address_space(3))) void *lds_ptr_t;
@@ -345,13 +386,79 @@ __device__ __forceinline__ float dpp_move(float v) {
 // tiles in LDS (one extra 128-bit LDS read and ~20 VALU instructions per wavefront and stage)
 // instead of by the pre-pass kernel: for the small blocks, whose launches are bound by latency,
 // this saves a launch and the global reads of the extension operands.
-template <int NWN, int WM, int MI, bool SWIGLU, bool RS>
+// The LoRA projection (and the extension operand) computed inside the launch that uses them: the
+// first `producers` blocks of the grid run lora_project_block (row tiles of 16 rows, K slices one
+// after the other) while the others multiply; a block of the product looks at its row tiles' words
+// behind its main loop -- long after they were raised -- and reads both operands with ordinary
+// loads (no cache on its die has seen those lines since the launch began).  The words live in
+// workspace that is all zero between launches (the region lora_tail.h describes: the tile words
+// from word kPrefillFoldTileWord of its first replica on); every block counts itself after its
+// look, on the replicated counts, and the last one zeroes words and counts.
+struct PrefillFold {
+    const uint16_t *a_cat;   // bf16 [r_total, K]
+    uint16_t *t;             // bf16 [M, RP], behind it the f32 tiles in which K slices meet
+    u32x4 *aext;             // the extension operand the producers write
+    float *partial;
+    int *counters;           // per row tile, zero on entry and exit (not the product's own counters)
+    unsigned *words;         // the zeroed region
+    int producers;           // row_tiles * kz rounded up to a multiple of 8 (the product's blocks keep their dies)
+    int row_tiles, kz, steps_per_slice;
+    int consumers;           // blocks of the product (grid padding included)
+    LoraScales ls;
+};
+constexpr int kPrefillFoldTileWord = 32;
+constexpr int kPrefillFoldMaxTiles = kLoraFoldReplicaWords - kPrefillFoldTileWord;
+constexpr int kPrefillFoldSpinLimit = 1 << 20;
+
+// rows [m0, m0 + rows) of T and of the extension operand are in memory
+__device__ __forceinline__ void prefill_fold_wait(const PrefillFold &pf, int m0, int rows, int lane) {
+    const int t0 = m0 >> 4, nt = min((rows + 15) >> 4, pf.row_tiles - t0);
+    for (int spins = 0; spins < kPrefillFoldSpinLimit; ++spins) {
+        unsigned f = 1u;
+        if (lane < nt) f = __hip_atomic_load(pf.words + kPrefillFoldTileWord + t0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (__builtin_amdgcn_ballot_w64(f == 0u) == 0) break;
+        __builtin_amdgcn_s_sleep(8);
+    }
+}
+// one wavefront of block `consumer`, after its look: count the block; the last one zeroes everything
+__device__ __forceinline__ void prefill_fold_done(const PrefillFold &pf, int consumer, int lane) {
+    const int replica = consumer % kLoraFoldReplicas;
+    const unsigned quota = (unsigned)(pf.consumers - replica + kLoraFoldReplicas - 1) / kLoraFoldReplicas;
+    const unsigned replicas = (unsigned)min(pf.consumers, kLoraFoldReplicas);
+    unsigned before = 0;
+    if (lane == 0)
+        before = __hip_atomic_fetch_add(pf.words + replica * kLoraFoldReplicaWords + kLoraFoldCountWord, 1u, __ATOMIC_RELAXED,
+                                        __HIP_MEMORY_SCOPE_AGENT);
+    before = (unsigned)__builtin_amdgcn_readfirstlane((int)before);
+    if (before != quota - 1u) return;
+    if (lane == 0) before = __hip_atomic_fetch_add(pf.words + kLoraFoldTopWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    before = (unsigned)__builtin_amdgcn_readfirstlane((int)before);
+    if (before != replicas - 1u) return;
+    for (int i = lane; i < pf.row_tiles; i += 64)
+        __hip_atomic_store(pf.words + kPrefillFoldTileWord + i, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane <= kLoraFoldTopWord)
+        for (int r = 0; r < kLoraFoldReplicas; ++r)
+            __hip_atomic_store(pf.words + r * kLoraFoldReplicaWords + lane, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int NWN, int WM, int MI, bool SWIGLU, bool RS, bool FOLD = false>
 __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void w4a16_prefill_kernel(
     const uint16_t *__restrict__ A, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C, const u32x4 *__restrict__ aext, int M, int N, int K, int Gs, int m_blocks,
     const uint16_t *__restrict__ lora_t, const uint16_t *__restrict__ lora_b, int r_total, int RP, int nb_full,
-    int KS, int GSb, float *partial, int *counters, int die_rows) {
+    int KS, int GSb, float *partial, int *counters, int die_rows, PrefillFold pf) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // the A ring; reused by the store
+    static_assert(!FOLD || (WM * NWN == 4 && !SWIGLU && !RS), "the projection's blocks have four wavefronts");
+    if constexpr (FOLD) {
+        if ((int)blockIdx.x < pf.producers) {
+            const int unit = blockIdx.x;
+            if (unit < pf.row_tiles * pf.kz)
+                lora_project_block<16>(lds, A, pf.a_cat, pf.t, M, K, r_total, RP, pf.steps_per_slice, pf.ls, pf.partial,
+                                       pf.counters, pf.aext, unit % pf.row_tiles, unit / pf.row_tiles, pf.kz,
+                                       pf.words + kPrefillFoldTileWord);
+            return;
+        }
+    }
     constexpr int BM = WM * MI * 32, BN = 64 * NWN;  // block rows and columns
     constexpr int NW = WM * NWN, NT = 64 * NW;       // wavefronts, threads
     constexpr int kAStageBytes = BM * 32 * 2;        // BM rows x 32 columns of bf16 per stage
@@ -380,6 +487,8 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     // where the loads that feed the matrix cores three stages ahead must hit) and
     // read each unit's weights from memory once.
     int id = blockIdx.x;
+    if constexpr (FOLD) id -= pf.producers;
+    [[maybe_unused]] const int consumer = id;
     const int n_blocks = N / BN;
     const int die_cols = 8 / die_rows, rows_per_die = m_blocks / die_rows;
     const int per_die_full = rows_per_die * ((nb_full + die_cols - 1) / die_cols);
@@ -389,7 +498,12 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     const int units_per_die = (units + die_cols - 1) / die_cols;
     const int die = id & 7, seq = id >> 3;
     const int unit = (die / die_rows) * units_per_die + seq / rows_per_die;
-    if (seq >= rows_per_die * units_per_die || unit >= units) return;  // grid padding (whole block, before any barrier)
+    if (seq >= rows_per_die * units_per_die || unit >= units) {  // grid padding (whole block, before any barrier)
+        if constexpr (FOLD) {
+            if (wave == 0) prefill_fold_done(pf, consumer, lane);  // counted like the others: it will never look
+        }
+        return;
+    }
     const int mb = (die % die_rows) * rows_per_die + seq % rows_per_die;
     int nb = unit, ks = 0;
     if (sliced) {
@@ -625,6 +739,11 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
 
     KILN_TL(1);
     if constexpr (RS) __syncthreads();  // every wavefront's row sums are in LDS
+    if constexpr (FOLD) {
+        // the rows of this block in the extension operand and in T: written during this launch
+        prefill_fold_wait(pf, m0, min(BM, M - m0), lane);
+        if (wave == 0) prefill_fold_done(pf, consumer, lane);
+    }
     // --- remove the 136 * sum(a) * scale surplus: extension contraction ------
     // Step e covers groups g_begin + 2e (lanes 0-31) and g_begin + 2e + 1 (lanes
     // 32-63), 8 slots each.  Operands come straight from global memory, loaded
@@ -878,6 +997,7 @@ size_t prefill_aext_bytes(int m, int k) { return (size_t)m * (k / kGroupK) * siz
 // ceil(256 / row tiles) slices per row tile: fewer than 256 + 2 x row tiles tiles of 64 or 16 rows
 // x 64 columns).
 constexpr int kProjectMaxCounters = 16384;
+constexpr int kProjectFoldCounters = 8192;  // folded into the product's launch: the product's counters first, then the projection's
 // measured at 2048 rows: 16-row blocks 9.9 us against 13.1 for K = 2560, 23.5 against 20.2 for K = 9216
 int lora_project_rows_per_block(int m, int k) { return m > 1024 && k > 4096 ? 64 : 16; }
 int prefill_lora_max_slices(int) { return 16; }
@@ -993,9 +1113,11 @@ namespace {
 constexpr int kMaxRowSumBytes = 24 * 1024;
 static int row_sum_bytes(int groups) { return groups * 64 * (int)sizeof(float); }
 
-template <int NWN, int WM, int MI, bool SWIGLU, bool RS>
+constexpr int kProjectLdsBytes16 = (16 + kProjectMaxRank) * kProjectRowBytes + kProjectMaxRank * (int)sizeof(float);
+
+template <int NWN, int WM, int MI, bool SWIGLU, bool RS, bool FOLD = false>
 hipError_t launch_shape_as(const PrefillArgs &a, int grid, int m_blocks, int RP, int KS, int GSb, int max_groups,
-                           hipStream_t stream) {
+                           hipStream_t stream, const PrefillFold &pf = PrefillFold{}) {
     constexpr int BM = WM * MI * 32, NW = WM * NWN;
     constexpr int kRing = kAStages * BM * 64;       // the A ring
     constexpr int kStore = NW * MI * 32 * 64 * 2;   // the store's per-wavefront transposes (reuses the ring)
@@ -1007,14 +1129,16 @@ hipError_t launch_shape_as(const PrefillArgs &a, int grid, int m_blocks, int RP,
     // The 256 x 128 block fits twice on a compute unit.  A grid of at most one block per unit
     // asks for more LDS than two blocks could share, so the dispatcher cannot stack two blocks
     // on one unit while others idle.
-    constexpr int kLdsSolo = (WM == 2 && NWN == 2) ? 96 * 1024 : kLdsMax;
-    const hipError_t attr = allow_dynamic_lds<&w4a16_prefill_kernel<NWN, WM, MI, SWIGLU, RS>>(kLdsSolo);
+    constexpr int kLdsSolo0 = (WM == 2 && NWN == 2) ? 96 * 1024 : kLdsMax;
+    constexpr int kLdsSolo = FOLD && kLdsSolo0 < kProjectLdsBytes16 ? kProjectLdsBytes16 : kLdsSolo0;
+    const hipError_t attr = allow_dynamic_lds<&w4a16_prefill_kernel<NWN, WM, MI, SWIGLU, RS, FOLD>>(kLdsSolo);
     if (attr != hipSuccess) return attr;
     if (WM == 2 && NWN == 2 && grid <= a.cus) lds_bytes = kLdsSolo;
-    w4a16_prefill_kernel<NWN, WM, MI, SWIGLU, RS><<<grid, 64 * NW, lds_bytes, stream>>>(
+    if (FOLD && lds_bytes < kProjectLdsBytes16) lds_bytes = kProjectLdsBytes16;  // the projection's blocks stage more
+    w4a16_prefill_kernel<NWN, WM, MI, SWIGLU, RS, FOLD><<<grid + (FOLD ? pf.producers : 0), 64 * NW, lds_bytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, (const u32x4 *)a.aext,
         a.M, a.N, a.K, a.Gs, m_blocks, (const uint16_t *)a.lora_t, (const uint16_t *)a.lora_b, a.r_total, RP,
-        a.nb_full, KS, GSb, a.partial, a.counters, prefill_die_rows(m_blocks));
+        a.nb_full, KS, GSb, a.partial, a.counters, prefill_die_rows(m_blocks), pf);
     return hipGetLastError();
 }
 
@@ -1042,6 +1166,25 @@ int lora_project_slices(int m, int k) {
     return kz < 1 ? 1 : kz;
 }
 
+// Many rows: rows per block, row tiles, K slices (as many as keep about 256 blocks busy) and steps of
+// 32 values per slice (whole groups).
+static void project_slicing(int m, int k, bool have_counters, int *rb_out, int *row_tiles_out, int *kz_out, int *per_slice_out) {
+    const int steps = k / 32;
+    const int rb = lora_project_rows_per_block(m, k), row_tiles = (m + rb - 1) / rb;
+    const int pieces = (k + kProjectPieceK - 1) / kProjectPieceK;
+    int kz = (256 + row_tiles - 1) / row_tiles;
+    const int zmax = rb == 16 ? 16 : 8;  // what the kernel's meeting reads in one go
+    if (kz > zmax) kz = zmax;
+    if (kz > pieces) kz = pieces;
+    if (row_tiles > kProjectMaxCounters || !have_counters) kz = 1;
+    const int per_slice = ((steps + kz - 1) / kz + 3) / 4 * 4;
+    kz = (steps + per_slice - 1) / per_slice;
+    *rb_out = rb;
+    *row_tiles_out = row_tiles;
+    *kz_out = kz;
+    *per_slice_out = per_slice;
+}
+
 hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t stream, int *slices, bool with_row_sums) {
     if (a.r_total < 1 || a.r_total > kProjectMaxRank || a.n_adapters < 1 || a.n_adapters > 8 || !a.lora_a ||
         !a.lora_t || !a.ranks || !a.scales || a.M < 1 || a.K < kGroupK)
@@ -1061,15 +1204,8 @@ hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t 
     if (with_row_sums && !aext) return hipErrorInvalidValue;
     if (!few_rows) {
         // many rows: T whole.  K slices that meet in f32 behind T, as many as keep about 256 blocks busy.
-        const int rb = lora_project_rows_per_block(a.M, a.K), row_tiles = (a.M + rb - 1) / rb;
-        const int pieces = (a.K + kProjectPieceK - 1) / kProjectPieceK;
-        int kz = (256 + row_tiles - 1) / row_tiles;
-        const int zmax = rb == 16 ? 16 : 8;  // what the kernel's meeting reads in one go
-        if (kz > zmax) kz = zmax;
-        if (kz > pieces) kz = pieces;
-        if (row_tiles > kProjectMaxCounters || !a.counters) kz = 1;
-        const int per_slice = ((steps + kz - 1) / kz + 3) / 4 * 4;
-        kz = (steps + per_slice - 1) / per_slice;
+        int rb, row_tiles, kz, per_slice;
+        project_slicing(a.M, a.K, a.counters != nullptr, &rb, &row_tiles, &kz, &per_slice);
         float *partial = reinterpret_cast<float *>(reinterpret_cast<char *>(a.lora_t) + (size_t)a.M * 64 * sizeof(uint16_t));
         const int lds_bytes = (rb + kProjectMaxRank) * kProjectRowBytes + kProjectMaxRank * (int)sizeof(float);
         if (rb == 16) {
@@ -1119,12 +1255,43 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         if (err != hipSuccess) return err;
     }
     int RP = 0;
+    // The projection inside the product's launch (PrefillFold): four-wavefront blocks, 16-row tiles of T,
+    // the extension operand from the projection, and room for its counters behind the product's.
+    PrefillFold pf{};
+    bool fold = false;
     if (a.r_total > 0) {
         RP = (a.r_total + 15) / 16 * 16;
-        int slices = 1;  // many rows: T is whole
-        err = launch_lora_project(a, false, stream, &slices, sums_with_projection);
-        if (err != hipSuccess) return err;
-        if (slices != 1) return hipErrorInvalidValue;
+        int rb = 0, row_tiles = 0, kz = 0, per_slice = 0;
+        project_slicing(a.M, a.K, a.counters != nullptr, &rb, &row_tiles, &kz, &per_slice);
+        const int sliced_tiles = (a.N / a.bn - a.nb_full) * ((a.M + a.bm - 1) / a.bm);
+        fold = a.lora_words && sums_with_projection && !a.swiglu && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
+               a.counters && row_tiles <= kPrefillFoldMaxTiles && row_tiles <= kProjectFoldCounters &&
+               sliced_tiles <= kProjectFoldCounters && a.n_adapters >= 1 && a.n_adapters <= 8 && a.lora_a && a.lora_t &&
+               a.ranks && a.scales && a.r_total <= kProjectMaxRank;
+        if (fold) {
+            pf.a_cat = (const uint16_t *)a.lora_a;
+            pf.t = (uint16_t *)a.lora_t;
+            pf.aext = (u32x4 *)a.aext;
+            pf.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(a.lora_t) + (size_t)a.M * 64 * sizeof(uint16_t));
+            pf.counters = a.counters + kProjectFoldCounters;
+            pf.words = a.lora_words;
+            pf.row_tiles = row_tiles;
+            pf.kz = kz;
+            pf.steps_per_slice = per_slice;
+            pf.producers = (row_tiles * kz + 7) / 8 * 8;
+            pf.ls.count = a.n_adapters;
+            int end = 0;
+            for (int i = 0; i < 8; ++i) {
+                if (i < a.n_adapters) end += a.ranks[i];
+                pf.ls.ends[i] = end;
+                pf.ls.scales[i] = i < a.n_adapters ? a.scales[i] : 0.f;
+            }
+        } else {
+            int slices = 1;  // many rows: T is whole
+            err = launch_lora_project(a, false, stream, &slices, sums_with_projection);
+            if (err != hipSuccess) return err;
+            if (slices != 1) return hipErrorInvalidValue;
+        }
     }
     if (a.bn != 128 && a.bn != 256) return hipErrorInvalidValue;
     if (a.swiglu && a.r_total > 0) return hipErrorInvalidValue;  // the LoRA term has no gate/up split
@@ -1139,6 +1306,11 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     shape.nb_full = a.nb_full;
     if (a.nb_full < 0 || a.nb_full > a.N / a.bn) return hipErrorInvalidValue;
     const int grid = prefill_grid(a.M, a.N, shape);
+    if (fold) {
+        pf.consumers = grid;
+        return a.bm == 64 ? launch_shape_as<4, 1, 2, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf)
+                          : launch_shape_as<4, 1, 4, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
+    }
     if (a.bm == 256) {
         return a.bn == 256 ? launch_shape<4, 2, 4>(a, grid, m_blocks, RP, KS, GSb, max_groups, rs, stream)
                            : launch_shape<2, 2, 4>(a, grid, m_blocks, RP, KS, GSb, max_groups, rs, stream);

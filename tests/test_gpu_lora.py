@@ -220,6 +220,54 @@ def test_adapters_with_zero_b_equal_the_plain_call_bit_for_bit(m, k, n):
     assert torch.equal(plain.view(torch.int16), with_adapters.view(torch.int16))
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (512, 2560, 18432),    # the benchmark's LoRA configuration: 64-row blocks, 32 row tiles x 7 K slices of the projection
+    (333, 2560, 18432),    # ragged last row tile
+    (1030, 2560, 8192),    # 128-row blocks
+])
+def test_projection_inside_the_matrix_core_launch(m, k, n):
+    """Where the product's blocks have four wavefronts and take the row sums from a pre-pass, the
+    projection (and those row sums) are computed by extra blocks of the product's own launch, which
+    raise a word per row tile in the zeroed workspace prefix.  Folded and in front must agree in every
+    bit; the prefix must be clean after every call; launches with alternating activations in a row
+    must each see their own T."""
+    from kiln_amd import _lib
+    L = _lib.load_tuning()
+    gen = torch.Generator(device="cuda").manual_seed(7 * m + k + n)
+    bt = torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device="cuda", generator=gen)
+    st = (torch.rand(k // 128, n, device="cuda", generator=gen) * 0.018 + 0.002).to(torch.float16)
+    xs = [(torch.randn(m, k, device="cuda", generator=gen) * 0.5).to(torch.bfloat16) for _ in range(2)]
+    ranks, scales = (16, 32), (0.5, 1.0)
+    a_cat = (torch.randn(sum(ranks), k, device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    b_cat = (torch.randn(n, sum(ranks), device="cuda", generator=gen) * 0.05).to(torch.bfloat16)
+    z = L.kiln_w4a16_workspace_zeroed_bytes()
+    ws = torch.empty(L.kiln_w4a16_workspace_bytes(m, n, k), dtype=torch.uint8, device="cuda")
+    ws[z:].fill_(0xA5)
+    ws[:z].zero_()
+    import ctypes
+    ranks_c = (ctypes.c_int * 2)(*ranks)
+    scales_c = (ctypes.c_float * 2)(*scales)
+
+    def call(x):
+        out = torch.full((m, n), float("nan"), dtype=torch.bfloat16, device="cuda")
+        rc = L.kiln_w4a16_gemm_lora(x.data_ptr(), bt.data_ptr(), out.data_ptr(), st.data_ptr(), m, n, k, ws.data_ptr(), 128,
+                                    torch.cuda.current_device(), torch.cuda.current_stream().cuda_stream,
+                                    a_cat.data_ptr(), b_cat.data_ptr(), sum(ranks), len(ranks), ranks_c, scales_c)
+        assert rc == _lib.OK, _lib.status_string(rc)
+        torch.cuda.synchronize()
+        assert int(ws[:z].count_nonzero()) == 0, "the call left words in the zeroed prefix"
+        return out
+
+    try:
+        L.kiln_w4a16_debug_lora_fold(0)
+        in_front = [call(x) for x in xs]
+        L.kiln_w4a16_debug_lora_fold(-1)
+        for i in range(40):
+            assert torch.equal(call(xs[i % 2]).view(torch.int16), in_front[i % 2].view(torch.int16)), i
+    finally:
+        L.kiln_w4a16_debug_lora_fold(-1)
+
+
 @pytest.mark.parametrize("m,k,n,ranks", [(200, 9216, 256, (7,)), (16, 9216, 2560, (16, 32))])
 def test_lora_run_to_run_determinism(oracle, m, k, n, ranks):
     """The projection's K slices meet as f32 tiles in the workspace (many rows) and the GEMM's own
