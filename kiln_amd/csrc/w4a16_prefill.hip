@@ -448,7 +448,7 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     const uint16_t *__restrict__ lora_t, const uint16_t *__restrict__ lora_b, int r_total, int RP, int nb_full,
     int KS, int GSb, float *partial, int *counters, int die_rows, PrefillFold pf) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // the A ring; reused by the store
-    static_assert(!FOLD || (WM * NWN == 4 && !SWIGLU && !RS), "the projection's blocks have four wavefronts");
+    static_assert(!FOLD || (WM * NWN == 4 && !SWIGLU), "the projection's blocks have four wavefronts");
     if constexpr (FOLD) {
         if ((int)blockIdx.x < pf.producers) {
             const int unit = blockIdx.x;
@@ -1256,7 +1256,8 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     }
     int RP = 0;
     // The projection inside the product's launch (PrefillFold): four-wavefront blocks, 16-row tiles of T,
-    // the extension operand from the projection, and room for its counters behind the product's.
+    // the extension operand from the projection (unless the blocks sum their rows themselves), and room
+    // for its counters behind the product's.
     PrefillFold pf{};
     bool fold = false;
     if (a.r_total > 0) {
@@ -1264,14 +1265,14 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         int rb = 0, row_tiles = 0, kz = 0, per_slice = 0;
         project_slicing(a.M, a.K, a.counters != nullptr, &rb, &row_tiles, &kz, &per_slice);
         const int sliced_tiles = (a.N / a.bn - a.nb_full) * ((a.M + a.bm - 1) / a.bm);
-        fold = a.lora_words && sums_with_projection && !a.swiglu && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
+        fold = a.lora_words && !a.swiglu && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
                a.counters && row_tiles <= kPrefillFoldMaxTiles && row_tiles <= kProjectFoldCounters &&
                sliced_tiles <= kProjectFoldCounters && a.n_adapters >= 1 && a.n_adapters <= 8 && a.lora_a && a.lora_t &&
                a.ranks && a.scales && a.r_total <= kProjectMaxRank;
         if (fold) {
             pf.a_cat = (const uint16_t *)a.lora_a;
             pf.t = (uint16_t *)a.lora_t;
-            pf.aext = (u32x4 *)a.aext;
+            pf.aext = rs ? nullptr : (u32x4 *)a.aext;  // blocks that sum their rows themselves need no operand
             pf.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(a.lora_t) + (size_t)a.M * 64 * sizeof(uint16_t));
             pf.counters = a.counters + kProjectFoldCounters;
             pf.words = a.lora_words;
@@ -1308,8 +1309,9 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     const int grid = prefill_grid(a.M, a.N, shape);
     if (fold) {
         pf.consumers = grid;
-        return a.bm == 64 ? launch_shape_as<4, 1, 2, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf)
-                          : launch_shape_as<4, 1, 4, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
+        if (a.bm == 128) return launch_shape_as<4, 1, 4, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
+        return rs ? launch_shape_as<4, 1, 2, false, true, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf)
+                  : launch_shape_as<4, 1, 2, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
     }
     if (a.bm == 256) {
         return a.bn == 256 ? launch_shape<4, 2, 4>(a, grid, m_blocks, RP, KS, GSb, max_groups, rs, stream)

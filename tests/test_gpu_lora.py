@@ -224,6 +224,8 @@ def test_adapters_with_zero_b_equal_the_plain_call_bit_for_bit(m, k, n):
     (512, 2560, 18432),    # the benchmark's LoRA configuration: 64-row blocks, 32 row tiles x 7 K slices of the projection
     (333, 2560, 18432),    # ragged last row tile
     (1030, 2560, 8192),    # 128-row blocks
+    (512, 9216, 2560),     # blocks that sum their rows themselves: the producers write T only
+    (300, 2560, 8192),     # likewise, ragged
 ])
 def test_projection_inside_the_matrix_core_launch(m, k, n):
     """Where the product's blocks have four wavefronts and take the row sums from a pre-pass, the
