@@ -105,6 +105,11 @@ struct MidArgs {
     bool swiglu;        // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
     bool flagged = false;  // KS > 1: `partial` is all zero between launches and the parts are their own arrival
                            // flags ((KS - 1) slices of mid_partial_bytes() / KS each); needs mid_flagged_ok()
+    // optional low-rank term (r_total == 0: none): C += lora_t * lora_b^T, r_total % 8 == 0, no swiglu
+    const void *lora_t = nullptr;  // bf16 [lora_slices][M][r_total rounded up to 16], written before this launch
+    const void *lora_b = nullptr;  // bf16 [N, r_total]
+    int r_total = 0;
+    int lora_slices = 1;
 };
 bool mid_flagged_ok(const MidArgs &a);
 int mid_column_blocks(const MidArgs &a);
@@ -112,6 +117,7 @@ int mid_max_rows_per_run();
 bool mid_plan_ok(const MidArgs &a);
 size_t mid_partial_bytes(const MidArgs &a);
 hipError_t launch_mid(const MidArgs &a, hipStream_t stream);
+hipError_t launch_mid_lora(const MidArgs &a, hipStream_t stream);  // its instances with the low-rank term (checked plan)
 
 // One launch of the prefill path (row-sum pre-pass + MFMA kernel), any M >= 1.
 struct PrefillArgs {

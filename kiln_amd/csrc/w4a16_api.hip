@@ -532,8 +532,9 @@ MidArgs mid_args(const MidPlan &mp, int m, int n, int k) {
 
 void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lora, GemmPlan *gp) {
     *gp = GemmPlan{};
-    // 33...128 rows of a plain GEMM: the mid-M kernel, one pass over the weights per 64 rows
-    if (!lora && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
+    // 33...128 rows: the mid-M kernel, one pass over the weights per 64 rows (with adapters whose
+    // stacked rank is a multiple of 8: the low-rank term is added from a projection launched in front)
+    if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
         (g_tune.mid == 1 ||
          (g_tune.prefill_min_m == 0 && m >= kMidMinM && m <= (n <= kMidNarrowN ? kMidMaxMNarrow : kMidMaxM)))) {
         const MidPlan mp = plan_mid(m, n, k, cus);
@@ -739,6 +740,25 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         ma.swiglu = swiglu;
         ma.counters = reinterpret_cast<int *>(workspace);
         ma.partial = reinterpret_cast<float *>(ws + wl.decode_partial);
+        if (lora) {  // the scaled projection of all rows onto the adapters, in K slices, ahead of the product
+            if (swiglu) return KILN_W4A16_ERR_KERN_SHAPE;
+            PrefillArgs pj{};
+            pj.A = A;
+            pj.M = prob_m;
+            pj.K = prob_k;
+            pj.lora_t = lora_t;
+            pj.lora_a = lora->a;
+            pj.r_total = lora->r_total;
+            pj.n_adapters = lora->n_adapters;
+            pj.ranks = lora->ranks;
+            pj.scales = lora->scales;
+            int slices = 1;
+            if (launch_lora_project(pj, true, st, &slices) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
+            ma.lora_t = lora_t;
+            ma.lora_b = lora->b;
+            ma.r_total = lora->r_total;
+            ma.lora_slices = slices;
+        }
         return launch_mid(ma, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
     }
 

@@ -33,8 +33,18 @@ namespace kiln {
 
 namespace {
 
+// This file is compiled twice: as it is for calls without adapters, and with -DKILN_MID_LORA=1 for calls
+// with them (launch_mid_lora only), so that what the low-rank term adds costs plain calls nothing.
+#ifndef KILN_MID_LORA
+#define KILN_MID_LORA 0
+#endif
+constexpr bool kMidLora = KILN_MID_LORA != 0;
+
 // Probe builds only (-DKILN_MID_TIMELINE): wall-clock stamps (100 MHz) per wavefront.
 #ifdef KILN_MID_TIMELINE
+#if KILN_MID_LORA
+#define g_mid_tl g_mid_tl_lora
+#endif
 __device__ long long *g_mid_tl;
 #define KILN_MID_TL(i) tl_[i] = (long long)__builtin_amdgcn_s_memrealtime()
 #else
@@ -98,11 +108,20 @@ struct MidScheduleOf {
     static constexpr MidSchedule value = mid_schedule(NG, NL, D);
 };
 
-template <int TP, int GPW>
+// The low-rank term of a call with adapters (LORA instances): T = the scaled projection of x onto the
+// stacked adapters in `slices` K slices, each rounded on its own, bf16 [slices][rows][rp] (written by
+// a launch in front of this one), B_cat bf16 [N][r_total], r_total % 8 == 0.
+struct MidLora {
+    const uint16_t *t;
+    const uint16_t *b;
+    int r_total, rp, slices;
+};
+
+template <int TP, int GPW, bool LORA>
 __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
-    int GS, int full_waves, int swiglu, int flagged, int col_shift) {
+    int GS, int full_waves, int swiglu, int flagged, int col_shift, MidLora lo) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     __shared__ int s_last;
     const int tid = threadIdx.x;
@@ -332,6 +351,37 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     };
     if (full) run(std::integral_constant<int, GPW>{});
     else if constexpr (GPW > 1) run(std::integral_constant<int, GPW - 1>{});
+    if constexpr (LORA) {
+        // y += T * B_cat^T (crates/kiln-model/src/lora_loader.rs:213-232, the second product) on the f32
+        // accumulators, before the single rounding: (K slice of T, 16 rank columns) pairs are dealt to the
+        // wavefronts of the first K slice's blocks, each adds its share to its own partial tiles, and
+        // the meeting below sums them with everything else.  Rows from M on read row M - 1 (never stored).
+        if (ks == 0) {
+            const int JS = lo.rp >> 4;
+            for (int c = wave; c < lo.slices * JS; c += nw) {
+                const int z = c / JS, j8 = (c - z * JS) * 16 + 8 * h;  // this lane's 8 rank columns
+                const bool live_rank = j8 + 8 <= lo.r_total;           // r_total % 8 == 0: all or none
+                u32x4 ta[2], tb[TP];
+#pragma unroll
+                for (int rb = 0; rb < 2; ++rb) {
+                    const int row = zr + min(32 * rb + l32, M - 1);
+                    ta[rb] = *reinterpret_cast<const u32x4 *>(lo.t + ((size_t)z * rows + row) * lo.rp + j8);
+                }
+#pragma unroll
+                for (int p = 0; p < TP; ++p) {
+                    const int col = min(tf + 2 * p, N / kTileN - 2) * kTileN + l32;
+                    tb[p] = u32x4{0u, 0u, 0u, 0u};
+                    if (live_rank) tb[p] = *reinterpret_cast<const u32x4 *>(lo.b + (size_t)col * lo.r_total + j8);
+                }
+#pragma unroll
+                for (int p = 0; p < TP; ++p)
+#pragma unroll
+                    for (int rb = 0; rb < 2; ++rb)
+                        acc[p][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ta[rb]),
+                                                                             __builtin_bit_cast(bf16x8, tb[p]), acc[p][rb], 0, 0, 0);
+            }
+        }
+    }
     KILN_MID_TL(5);  // main loop done
 
     // --- the wavefronts' partial tiles meet in LDS, at most two pairs at a time (a wavefront's
@@ -495,16 +545,17 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
 
 template <int TP, int GPW>
 hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
-    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW>>(kMidWaves * kMidSlotBytes);
+    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora>>(kMidWaves * kMidSlotBytes);
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
     const int full_waves = a.GS - a.waves * (GPW - 1);
-    w4a16_mid_kernel<TP, GPW><<<dim3((NT + 2 * TP - 1) / (2 * TP), a.KS, runs), a.waves * 64, a.waves * kMidSlotBytes,
-                               stream>>>(
+    const MidLora lo{(const uint16_t *)a.lora_t, (const uint16_t *)a.lora_b, a.r_total, (a.r_total + 15) / 16 * 16, a.lora_slices};
+    w4a16_mid_kernel<TP, GPW, kMidLora><<<dim3((NT + 2 * TP - 1) / (2 * TP), a.KS, runs), a.waves * 64,
+                                         a.waves * kMidSlotBytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
         a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
-        a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0);
+        a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0, lo);
     return hipGetLastError();
 }
 
@@ -521,6 +572,19 @@ hipError_t launch_mid_t(const MidArgs &a, int gpw, hipStream_t stream) {
 
 }  // namespace
 
+#if KILN_MID_LORA
+// The instances with the low-rank term; the caller (launch_mid) has checked the plan.
+hipError_t launch_mid_lora(const MidArgs &a, hipStream_t stream) {
+    if (a.r_total < 8 || a.r_total > 64 || a.r_total % 8 != 0 || !a.lora_t || !a.lora_b || a.lora_slices < 1 || a.swiglu)
+        return hipErrorInvalidValue;
+    const int gpw = (a.GS + a.waves - 1) / a.waves;
+    switch (a.pairs) {
+        case 1: return launch_mid_t<1>(a, gpw, stream);
+        case 2: return launch_mid_t<2>(a, gpw, stream);
+        default: return launch_mid_t<3>(a, gpw, stream);
+    }
+}
+#else
 int mid_max_rows_per_run() { return kMidRows; }
 
 // What a launch of the mid-M kernel assumes: one to three pairs of tiles per block (N % 256 == 0
@@ -553,6 +617,7 @@ hipError_t launch_mid(const MidArgs &a, hipStream_t stream) {
     if (!mid_plan_ok(a)) return hipErrorInvalidValue;
     if (a.KS > 1 && (!a.partial || !a.counters)) return hipErrorInvalidValue;
     if (a.flagged && !mid_flagged_ok(a)) return hipErrorInvalidValue;
+    if (a.r_total > 0) return launch_mid_lora(a, stream);
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.pairs) {
         case 1: return launch_mid_t<1>(a, gpw, stream);
@@ -560,11 +625,16 @@ hipError_t launch_mid(const MidArgs &a, hipStream_t stream) {
         default: return launch_mid_t<3>(a, gpw, stream);
     }
 }
+#endif  // KILN_MID_LORA
 
 }  // namespace kiln
 
 #ifdef KILN_MID_TIMELINE
+#if KILN_MID_LORA
+extern "C" int kiln_mid_timeline_lora(long long *buf) {
+#else
 extern "C" int kiln_mid_timeline(long long *buf) {
+#endif
     return (int)hipMemcpyToSymbol(HIP_SYMBOL(kiln::g_mid_tl), &buf, sizeof(buf));
 }
 #endif
