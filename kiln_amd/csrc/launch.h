@@ -110,6 +110,15 @@ struct MidArgs {
     const void *lora_b = nullptr;  // bf16 [N, r_total]
     int r_total = 0;
     int lora_slices = 1;
+    // lora_producers > 0: the projection runs in this launch's first blocks (16-row tiles x lora_slices K slices of
+    // lora_steps_per_slice steps) and lora_t is written here; needs >= 4 wavefronts per block
+    int lora_producers = 0;
+    int lora_steps_per_slice = 0;
+    const void *lora_a = nullptr;    // bf16 [r_total, K]
+    unsigned *lora_words = nullptr;  // 64 KiB that are zero between launches (lora_tail.h)
+    int lora_adapters = 0;           // 1...8
+    int lora_ends[8] = {};           // exclusive end column of adapter i on the stacked rank axis
+    float lora_scales[8] = {};
 };
 bool mid_flagged_ok(const MidArgs &a);
 int mid_column_blocks(const MidArgs &a);

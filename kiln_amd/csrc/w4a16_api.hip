@@ -537,7 +537,9 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
     if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
         (g_tune.mid == 1 ||
          (g_tune.prefill_min_m == 0 && m >= kMidMinM && m <= (n <= kMidNarrowN ? kMidMaxMNarrow : kMidMaxM)))) {
-        const MidPlan mp = plan_mid(m, n, k, cus);
+        // with adapters the projection runs in the launch's first blocks: plan for the chip less those
+        const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
+        const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus);
         if (mp.ok) {
             gp->mid = true;
             gp->mp = mp;
@@ -740,8 +742,33 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         ma.swiglu = swiglu;
         ma.counters = reinterpret_cast<int *>(workspace);
         ma.partial = reinterpret_cast<float *>(ws + wl.decode_partial);
-        if (lora) {  // the scaled projection of all rows onto the adapters, in K slices, ahead of the product
+        if (lora) {  // the scaled projection of all rows onto the adapters, in K slices
             if (swiglu) return KILN_W4A16_ERR_KERN_SHAPE;
+            ma.lora_t = lora_t;
+            ma.lora_b = lora->b;
+            ma.r_total = lora->r_total;
+            // ... inside the product's launch where its blocks have the threads for it and all blocks fit the chip
+            const int steps = prob_k / 32, row_tiles = ceil_div(prob_m, 16);
+            int kz = lora_project_slices(prob_m, prob_k);
+            const int per_slice = ((steps + kz - 1) / kz + 3) / 4 * 4;  // whole 128-value groups
+            kz = (steps + per_slice - 1) / per_slice;
+            const int runs = ceil_div(prob_m, mid_max_rows_per_run());
+            if (g_tune.lora_fold != 0 && ma.waves >= 4 && lora->n_adapters <= 8 &&
+                mid_column_blocks(ma) * ma.KS * runs + row_tiles * kz <= cus) {
+                ma.lora_slices = kz;
+                ma.lora_producers = row_tiles * kz;
+                ma.lora_steps_per_slice = per_slice;
+                ma.lora_a = lora->a;
+                ma.lora_words = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
+                ma.lora_adapters = lora->n_adapters;
+                int end = 0;
+                for (int i = 0; i < 8; ++i) {
+                    if (i < lora->n_adapters) end += lora->ranks[i];
+                    ma.lora_ends[i] = end;
+                    ma.lora_scales[i] = i < lora->n_adapters ? lora->scales[i] : 0.f;
+                }
+                return launch_mid(ma, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+            }
             PrefillArgs pj{};
             pj.A = A;
             pj.M = prob_m;
@@ -754,9 +781,6 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             pj.scales = lora->scales;
             int slices = 1;
             if (launch_lora_project(pj, true, st, &slices) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
-            ma.lora_t = lora_t;
-            ma.lora_b = lora->b;
-            ma.r_total = lora->r_total;
             ma.lora_slices = slices;
         }
         return launch_mid(ma, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;

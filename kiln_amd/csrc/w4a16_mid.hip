@@ -28,6 +28,8 @@
 // order; K slices of a tile meet in the workspace, last arriver adds in slice order.
 #include "async_loads.h"
 #include "launch.h"
+#include "lora_project.h"
+#include "lora_tail.h"
 
 namespace kiln {
 
@@ -115,7 +117,18 @@ struct MidLora {
     const uint16_t *t;
     const uint16_t *b;
     int r_total, rp, slices;
+    // producers > 0: the projection runs in this launch's first `producers` blocks (row tiles of 16 rows x
+    // the K slices, lora_project_block), which raise a word per (slice, row tile) -- in 16 copies, 4 KiB
+    // apart, block b looks at copy b % 16: hundreds of readers of one address are served one by one -- in
+    // workspace that is zero between launches; the blocks of the first K slice look at the words of their
+    // rows behind their main loop, count themselves, and the last one zeroes words and counts.
+    const uint16_t *a_cat;
+    unsigned *words;
+    int producers, row_tiles, steps_per_slice, col_blocks, consumers;
+    LoraScales ls;
 };
+constexpr int kMidFoldTileWord = 32;  // a copy's words start here (the first words are the small-M kernel's)
+constexpr int kMidFoldSpinLimit = 1 << 20;
 
 template <int TP, int GPW, bool LORA>
 __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
@@ -145,18 +158,40 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     } timeline_writer{tl_, lane, wave};
 #endif
     KILN_MID_TL(0);
-    // blockIdx.z: which run of 64 rows (each with its own counters and partial tiles)
-    const int zr = blockIdx.z * kMidRows;
+    // Grid (column blocks, K slices, runs of 64 rows) -- or, with the projection in this launch, one row
+    // of blocks: the producers, then the same order.
+    int bx = blockIdx.x, by = blockIdx.y, bz = blockIdx.z, ncb = gridDim.x;
+    if constexpr (LORA) {
+        if (lo.producers > 0) {
+            int id = blockIdx.x;
+            if (id < lo.producers) {
+                const int tile = id % lo.row_tiles, slice = id / lo.row_tiles;
+                lora_project_block<16>(lds, A_all, lo.a_cat, const_cast<uint16_t *>(lo.t), rows, K, lo.r_total, lo.rp,
+                                       lo.steps_per_slice, lo.ls, nullptr, nullptr, nullptr, tile, slice, lo.slices,
+                                       lo.words + kMidFoldTileWord + slice * lo.row_tiles, kLoraFoldReplicas,
+                                       kLoraFoldReplicaWords);
+                return;
+            }
+            id -= lo.producers;
+            ncb = lo.col_blocks;
+            bx = id % ncb;
+            id /= ncb;
+            by = id % KS;
+            bz = id / KS;
+        }
+    }
+    // bz: which run of 64 rows (each with its own counters and partial tiles)
+    const int zr = bz * kMidRows;
     const int M = min(rows - zr, kMidRows);
     const uint16_t *__restrict__ A = A_all + (size_t)zr * K;
     const int ldc = swiglu ? N >> 1 : N;  // the fused gate/up result is half as wide
     uint16_t *__restrict__ C = C_all + (size_t)zr * ldc;
-    const int ks = blockIdx.y;
+    const int ks = by;
     // Column block of this block.  Blocks go to the eight dies round-robin by linear index; the
     // counter-free exchange shifts the column block by col_shift per slice so that the slices of a
     // tile sit on different dies (a device-scope store and the device-scope load that polls it
     // are slow when they meet in one die's L2).
-    const int cb = (int)((blockIdx.x + ks * col_shift) % gridDim.x);
+    const int cb = (bx + ks * col_shift) % ncb;
     const int tf = cb * (2 * TP);  // first 16-column tile of the block
     // the first `full_waves` wavefronts own GPW groups each, the others GPW - 1
     const bool full = wave < full_waves;
@@ -356,6 +391,47 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         // accumulators, before the single rounding: (K slice of T, 16 rank columns) pairs are dealt to the
         // wavefronts of the first K slice's blocks, each adds its share to its own partial tiles, and
         // the meeting below sums them with everything else.  Rows from M on read row M - 1 (never stored).
+        if (ks == 0 && lo.producers > 0) {
+            // T of this run's rows, every slice: one wavefront looks (lane 4 z + i: slice z, i-th row tile
+            // of the run), counts the block, and the barrier tells the others
+            if (wave == 0) {
+                const int t0 = zr >> 4, nt = min((M + 15) >> 4, lo.row_tiles - t0), consumer = bz * ncb + bx;
+                const unsigned *mine = lo.words + (consumer % kLoraFoldReplicas) * kLoraFoldReplicaWords + kMidFoldTileWord;
+                for (int spins = 0; spins < kMidFoldSpinLimit; ++spins) {
+                    unsigned f = 1u;
+                    if ((lane >> 2) < lo.slices && (lane & 3) < nt)
+                        f = __hip_atomic_load(mine + (lane >> 2) * lo.row_tiles + t0 + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (__builtin_amdgcn_ballot_w64(f == 0u) == 0) break;
+                    __builtin_amdgcn_s_sleep(4);
+                }
+                // count: the replica's count, then the top count; the last block zeroes words and counts
+                const int replica = consumer % kLoraFoldReplicas;
+                const unsigned quota = (unsigned)(lo.consumers - replica + kLoraFoldReplicas - 1) / kLoraFoldReplicas;
+                const unsigned replicas = (unsigned)min(lo.consumers, kLoraFoldReplicas);
+                unsigned before = 0;
+                if (lane == 0)
+                    before = __hip_atomic_fetch_add(lo.words + replica * kLoraFoldReplicaWords + kLoraFoldCountWord, 1u,
+                                                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                bool last = (unsigned)__builtin_amdgcn_readfirstlane((int)before) == quota - 1u;
+                if (last) {
+                    if (lane == 0)
+                        before = __hip_atomic_fetch_add(lo.words + kLoraFoldTopWord, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    last = (unsigned)__builtin_amdgcn_readfirstlane((int)before) == replicas - 1u;
+                }
+                if (last) {
+                    const int n_words = lo.slices * lo.row_tiles;
+                    for (int r = 0; r < kLoraFoldReplicas; ++r) {
+                        for (int i = lane; i < n_words; i += 64)
+                            __hip_atomic_store(lo.words + r * kLoraFoldReplicaWords + kMidFoldTileWord + i, 0u, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                        if (lane <= kLoraFoldTopWord)
+                            __hip_atomic_store(lo.words + r * kLoraFoldReplicaWords + lane, 0u, __ATOMIC_RELAXED,
+                                               __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
+            }
+            __syncthreads();
+        }
         if (ks == 0) {
             const int JS = lo.rp >> 4;
             for (int c = wave; c < lo.slices * JS; c += nw) {
@@ -420,8 +496,8 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                 }
         }
     };
-    float *partial = partial_all + ((size_t)(blockIdx.z * KS) * gridDim.x + cb) * (kItems * 256);
-    const size_t slice_stride = (size_t)gridDim.x * (kItems * 256);  // floats between two K slices of a block
+    float *partial = partial_all + ((size_t)(bz * KS) * ncb + cb) * (kItems * 256);
+    const size_t slice_stride = (size_t)ncb * (kItems * 256);  // floats between two K slices of a block
     f32x4 *mine = reinterpret_cast<f32x4 *>(slot);
     // item `local` of the phase, summed over the wavefronts in wavefront (= ascending K) order
     auto sum_over_wavefronts = [&](int local) {
@@ -522,7 +598,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     // adds the slices in ascending K order and leaves the counter zero.
     wait_vector_loads<0>();
     __syncthreads();
-    int *counter = counters_all + blockIdx.z * gridDim.x + blockIdx.x;
+    int *counter = counters_all + bz * ncb + bx;
     if (tid == 0) {
         const bool last = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == KS - 1;
         s_last = last;
@@ -550,9 +626,30 @@ hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
     const int full_waves = a.GS - a.waves * (GPW - 1);
-    const MidLora lo{(const uint16_t *)a.lora_t, (const uint16_t *)a.lora_b, a.r_total, (a.r_total + 15) / 16 * 16, a.lora_slices};
-    w4a16_mid_kernel<TP, GPW, kMidLora><<<dim3((NT + 2 * TP - 1) / (2 * TP), a.KS, runs), a.waves * 64,
-                                         a.waves * kMidSlotBytes, stream>>>(
+    MidLora lo{};
+    lo.t = (const uint16_t *)a.lora_t;
+    lo.b = (const uint16_t *)a.lora_b;
+    lo.r_total = a.r_total;
+    lo.rp = (a.r_total + 15) / 16 * 16;
+    lo.slices = a.lora_slices;
+    const int col_blocks = (NT + 2 * TP - 1) / (2 * TP);
+    dim3 grid(col_blocks, a.KS, runs);
+    if (a.lora_producers > 0) {
+        lo.a_cat = (const uint16_t *)a.lora_a;
+        lo.words = a.lora_words;
+        lo.producers = a.lora_producers;
+        lo.row_tiles = (a.M + 15) / 16;
+        lo.steps_per_slice = a.lora_steps_per_slice;
+        lo.col_blocks = col_blocks;
+        lo.consumers = col_blocks * runs;
+        lo.ls.count = a.lora_adapters;
+        for (int i = 0; i < 8; ++i) {
+            lo.ls.ends[i] = a.lora_ends[i];
+            lo.ls.scales[i] = a.lora_scales[i];
+        }
+        grid = dim3(a.lora_producers + col_blocks * a.KS * runs, 1, 1);
+    }
+    w4a16_mid_kernel<TP, GPW, kMidLora><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
         a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
         a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0, lo);
@@ -577,6 +674,15 @@ hipError_t launch_mid_t(const MidArgs &a, int gpw, hipStream_t stream) {
 hipError_t launch_mid_lora(const MidArgs &a, hipStream_t stream) {
     if (a.r_total < 8 || a.r_total > 64 || a.r_total % 8 != 0 || !a.lora_t || !a.lora_b || a.lora_slices < 1 || a.swiglu)
         return hipErrorInvalidValue;
+    if (a.lora_producers > 0) {
+        // the projection's blocks: 256 working threads, 16-row tiles, words for (slice, tile) in a copy's 4 KiB
+        const int row_tiles = (a.M + 15) / 16;
+        if (a.waves < 4 || a.lora_slices > 16 || row_tiles * a.lora_slices > kLoraFoldReplicaWords - kMidFoldTileWord ||
+            a.lora_producers != row_tiles * a.lora_slices || !a.lora_a || !a.lora_words || a.lora_adapters < 1 ||
+            a.lora_adapters > 8 || a.lora_steps_per_slice < 4 || a.lora_steps_per_slice % 4 != 0 ||
+            (long)a.lora_slices * a.lora_steps_per_slice * 32 < a.K || a.M > 4 * kMidRows)
+            return hipErrorInvalidValue;
+    }
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.pairs) {
         case 1: return launch_mid_t<1>(a, gpw, stream);

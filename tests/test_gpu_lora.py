@@ -226,10 +226,14 @@ def test_adapters_with_zero_b_equal_the_plain_call_bit_for_bit(m, k, n):
     (1030, 2560, 8192),    # 128-row blocks
     (512, 9216, 2560),     # blocks that sum their rows themselves: the producers write T only
     (300, 2560, 8192),     # likewise, ragged
+    (64, 4096, 2560),      # the mid-M kernel: producers of 256 working threads in blocks of 512, T in K slices
+    (33, 2560, 18432),     # ... three tile pairs per block, a ragged run
+    (100, 2560, 8192),     # ... two runs of 64 rows
+    (48, 9216, 2560),      # ... K slices of the product and of the projection
 ])
 def test_projection_inside_the_matrix_core_launch(m, k, n):
-    """Where the product's blocks have four wavefronts and take the row sums from a pre-pass, the
-    projection (and those row sums) are computed by extra blocks of the product's own launch, which
+    """Beyond 32 rows the projection (on the matrix-core path also the row sums, where they come from a
+    pre-pass) is computed by extra blocks of the product's own launch where the block shape allows it; they
     raise a word per row tile in the zeroed workspace prefix.  Folded and in front must agree in every
     bit; the prefix must be clean after every call; launches with alternating activations in a row
     must each see their own T."""
