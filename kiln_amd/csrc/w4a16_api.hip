@@ -465,8 +465,11 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // against 9.1 / 10.8 / 14.1 / 14.1) and up to two runs of 64 -- three for outputs of up to 8192
 // columns, where it still leads the matrix-core kernel's 64-row blocks at 192 rows (21.3 against
 // 23.8 us on the in-projection, 12.0 against 21.0 on the out-projection) while the widest
-// projection does not (38.8 against 34.5).
-constexpr int kMidMinM = 33, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN = 8192;
+// projection does not (38.8 against 34.5).  With adapters it starts at 17 rows: the two-slab
+// instance needs the projection from a launch in front, the mid-M kernel computes it in its own
+// first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.2 / 12.8 /
+// 16.5 / 16.3 us against 14.4 / 13.3 / 19.2 / 17.0).
+constexpr int kMidMinM = 33, kMidMinMLora = 17, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN = 8192;
 
 // Do the K slices of this mid-M launch meet in the zeroed region, the parts being their own arrival flags?
 bool mid_flagged(const MidArgs &a) {
@@ -536,7 +539,7 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
     // stacked rank is a multiple of 8: the low-rank term is added from a projection launched in front)
     if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
         (g_tune.mid == 1 ||
-         (g_tune.prefill_min_m == 0 && m >= kMidMinM && m <= (n <= kMidNarrowN ? kMidMaxMNarrow : kMidMaxM)))) {
+         (g_tune.prefill_min_m == 0 && m >= (lora ? kMidMinMLora : kMidMinM) && m <= (n <= kMidNarrowN ? kMidMaxMNarrow : kMidMaxM)))) {
         // with adapters the projection runs in the launch's first blocks: plan for the chip less those
         const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
         const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus);

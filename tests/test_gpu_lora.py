@@ -46,8 +46,8 @@ def test_fused_lora_matches_oracle(oracle, m, k, n, ranks, scales):
 @pytest.mark.parametrize("k,n", [(2560, 18432), (9216, 2560), (2560, 8192)])
 @pytest.mark.parametrize("m", [1, 3, 16, 17, 32, 33, 48, 64, 80])
 def test_lora_on_few_rows(oracle, m, k, n):
-    """Few rows take the small-M kernels, which add the low-rank term where they store a tile:
-    one launch up to 32 rows, slabs beyond; adapters large enough that a missing term fails."""
+    """Few rows take the small-M kernels, which add the low-rank term where they store a tile (the
+    decode kernel up to 16 rows, the mid-M kernel beyond); adapters large enough that a missing term fails."""
     _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=3 * m + n, sigma_ab=0.05)
 
 
@@ -230,9 +230,11 @@ def test_adapters_with_zero_b_equal_the_plain_call_bit_for_bit(m, k, n):
     (33, 2560, 18432),     # ... three tile pairs per block, a ragged run
     (100, 2560, 8192),     # ... two runs of 64 rows
     (48, 9216, 2560),      # ... K slices of the product and of the projection
+    (17, 4096, 2560),      # ... which calls with adapters take from 17 rows on
+    (24, 2560, 18432),
 ])
 def test_projection_inside_the_matrix_core_launch(m, k, n):
-    """Beyond 32 rows the projection (on the matrix-core path also the row sums, where they come from a
+    """Beyond 16 rows the projection (on the matrix-core path also the row sums, where they come from a
     pre-pass) is computed by extra blocks of the product's own launch where the block shape allows it; they
     raise a word per row tile in the zeroed workspace prefix.  Folded and in front must agree in every
     bit; the prefix must be clean after every call; launches with alternating activations in a row
