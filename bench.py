@@ -250,11 +250,17 @@ def main() -> int:
                   for name, kn in shapes.items()}
             x512 = torch.randn(512, 2560, device=dev).to(torch.bfloat16)
             o512 = torch.empty(512, 18432, dtype=torch.bfloat16, device=dev)
+            x64 = {name: torch.randn(64, kn[0], device=dev).to(torch.bfloat16) for name, kn in shapes.items()}
+            o64 = {name: torch.empty(64, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in shapes.items()}
             for i in range(args.steps):
                 for name in shapes:
                     b, s = layers[i % LAYERS][name]
                     marlin_gemm.marlin_w4a16_gemm_lora(x[name], b, s, GROUP, ad[name][0], ad[name][1], ranks,
                                                        lscales, out=out[name])
+                for name in shapes:
+                    b, s = layers[i % LAYERS][name]
+                    marlin_gemm.marlin_w4a16_gemm_lora(x64[name], b, s, GROUP, ad[name][0], ad[name][1], ranks,
+                                                       lscales, out=o64[name])
                 b, s = layers[i % LAYERS]["gate_up"]
                 marlin_gemm.marlin_w4a16_gemm_lora(x512, b, s, GROUP, ad["gate_up"][0], ad["gate_up"][1], ranks,
                                                    lscales, out=o512)
