@@ -158,6 +158,26 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu(
 size_t kiln_w4a16_swiglu_workspace_bytes(int prob_m, int n_out, int prob_k);
 
 /*
+ * kiln_w4a16_gemm_swiglu with LoRA adapters on gate_proj and up_proj:
+ * C[m, n_out] = silu(gate + d_gate) * (up + d_up), d = the low-rank terms of kiln_w4a16_gemm_lora.
+ * The reference adds each projection's delta to its bf16 GEMM result before silu and the multiply
+ * (mlp_proj_forward with lora_layer.gate_proj / up_proj, crates/kiln-model/src/forward.rs:2771-2819);
+ * here the deltas land on the f32 sums and the product is rounded once.
+ *   lora_a  bf16 [r_total, k]           A matrices of gate's adapters, then of up's, row-concatenated
+ *   lora_b  bf16 [2 * n_out, r_total]   rows in the packed column order (per 16 rows: 8 gate columns,
+ *           then the 8 matching up columns); a gate row holds gate's B entries in the rank columns of
+ *           gate's adapters and zeros in up's, an up row the reverse
+ *   ranks, scales: one entry per stacked adapter (gate's first), sum(ranks) == r_total <= 64.
+ * Workspace: kiln_w4a16_swiglu_workspace_bytes(m, n_out, k).
+ */
+kiln_marlin_status_t kiln_w4a16_gemm_swiglu_lora(
+    const void *A, const void *B, void *C, const void *s,
+    int prob_m, int n_out, int prob_k,
+    void *workspace, int groupsize, int dev, void *stream,
+    const void *lora_a, const void *lora_b, int r_total,
+    int n_adapters, const int *ranks, const float *scales);
+
+/*
  * out[k, n] (f32, row-major) = (code - 8) * f32(scale), read from the tile
  * layout on the device.  The device-side statement of lib.rs:425; used to
  * prove the repack bit-exact.  No counterpart entry point in the reference.

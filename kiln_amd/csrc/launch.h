@@ -105,7 +105,8 @@ struct MidArgs {
     bool swiglu;        // columns are gate/up interleaved by 8 inside every tile; C is [M, N/2] = silu(gate) * up
     bool flagged = false;  // KS > 1: `partial` is all zero between launches and the parts are their own arrival
                            // flags ((KS - 1) slices of mid_partial_bytes() / KS each); needs mid_flagged_ok()
-    // optional low-rank term (r_total == 0: none): C += lora_t * lora_b^T, r_total % 8 == 0, no swiglu
+    // optional low-rank term (r_total == 0: none): C += lora_t * lora_b^T, r_total % 8 == 0
+    // (with swiglu the rows of lora_b are in the packed column order)
     const void *lora_t = nullptr;  // bf16 [lora_slices][M][r_total rounded up to 16], written before this launch
     const void *lora_b = nullptr;  // bf16 [N, r_total]
     int r_total = 0;

@@ -948,7 +948,6 @@ hipError_t launch_decode(const DecodeArgs &a, hipStream_t stream) {
     const int gs_last = G - (a.KS - 1) * a.GS;  // smallest slice
     const bool sane = a.waves >= 1 && a.waves <= kMaxWaves && a.M >= 1 && a.U >= 1 && a.GS >= 1 && a.KS >= 1;
     if (a.r_total < 0 || a.r_total > 64) return hipErrorInvalidValue;
-    if (a.swiglu && a.r_total > 0) return hipErrorInvalidValue;  // the low-rank term has no gate/up split
     if (a.r_total > 0 && (!a.lora_t || !a.lora_b || a.lora_slices < 1 || a.lora_rows < a.M)) return hipErrorInvalidValue;
     if (a.rows > a.M && (!a.regs || a.M != 32 || a.rows > 128)) return hipErrorInvalidValue;  // up to four runs of 32 rows
     if (a.regs) {

@@ -654,9 +654,10 @@ bool decode_gmp_ok(const DecodeArgs &a) {
     const int G = a.K / kGroupK;
     if (a.M < 1 || a.M > 16 || a.gm_tiles < 1 || a.gm_tiles > 6) return false;
     if (a.r_total > 0) {
-        // the low-rank term has no gate/up split; its operands are read from LDS in 16-byte pieces by one
-        // wavefront more than the main loop uses; T is whole and belongs to exactly this launch's rows
-        if (a.swiglu || a.r_total > 64 || a.r_total % 8 != 0 || a.waves + 1 > kGmpMaxWaves) return false;
+        // the low-rank term's operands are read from LDS in 16-byte pieces by one wavefront more than the
+        // main loop uses; T is whole and belongs to exactly this launch's rows (with the fused gate/up
+        // store the rows of lora_b are in the packed column order, so nothing changes here)
+        if (a.r_total > 64 || a.r_total % 8 != 0 || a.waves + 1 > kGmpMaxWaves) return false;
         if (a.lora_slices < 1 || a.lora_slices > 16 || a.lora_rows != a.M || !a.lora_t || !a.lora_b) return false;
     }
     if (a.KS < 1 || a.GS < 1 || a.KS * a.GS != G || a.waves < 1 || a.waves > kGmpMaxWaves || a.waves > a.GS) return false;

@@ -672,7 +672,7 @@ hipError_t launch_mid_t(const MidArgs &a, int gpw, hipStream_t stream) {
 #if KILN_MID_LORA
 // The instances with the low-rank term; the caller (launch_mid) has checked the plan.
 hipError_t launch_mid_lora(const MidArgs &a, hipStream_t stream) {
-    if (a.r_total < 8 || a.r_total > 64 || a.r_total % 8 != 0 || !a.lora_t || !a.lora_b || a.lora_slices < 1 || a.swiglu)
+    if (a.r_total < 8 || a.r_total > 64 || a.r_total % 8 != 0 || !a.lora_t || !a.lora_b || a.lora_slices < 1)
         return hipErrorInvalidValue;
     if (a.lora_producers > 0) {
         // the projection's blocks: 256 working threads, 16-row tiles, words for (slice, tile) in a copy's 4 KiB

@@ -198,7 +198,7 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     const uint16_t *__restrict__ lora_t, const uint16_t *__restrict__ lora_b, int r_total, int RP, int nb_full,
     int KS, int GSb, float *partial, int *counters, int die_rows, PrefillFold pf) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];  // the A ring; reused by the store
-    static_assert(!FOLD || (WM * NWN == 4 && !SWIGLU), "the projection's blocks have four wavefronts");
+    static_assert(!FOLD || WM * NWN == 4, "the projection's blocks have four wavefronts");
     if constexpr (FOLD) {
         if ((int)blockIdx.x < pf.producers) {
             const int unit = blockIdx.x;
@@ -601,7 +601,10 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
         bf16x8 lb[2];
 #pragma unroll
         for (int ni = 0; ni < 2; ++ni) {
-            const uint16_t *bp = lora_b + (size_t)(n0 + wn * 64 + ni * 32 + l32) * r_total + j8;
+            // the lane's column of accumulator ni, as the main loop maps it (SWIGLU: gate columns of four
+            // tiles in accumulator 0, their up columns in 1; lora_b's rows are in the packed column order)
+            const int bcol = SWIGLU ? 16 * (l32 >> 3) + 8 * ni + (l32 & 7) : ni * 32 + l32;
+            const uint16_t *bp = lora_b + (size_t)(n0 + wn * 64 + bcol) * r_total + j8;
             if ((r_total & 7) == 0 && j8 + 8 <= r_total) {
                 lb[ni] = *reinterpret_cast<const bf16x8 *>(bp);
             } else {
@@ -1015,7 +1018,7 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         int rb = 0, row_tiles = 0, kz = 0, per_slice = 0;
         project_slicing(a.M, a.K, a.counters != nullptr, &rb, &row_tiles, &kz, &per_slice);
         const int sliced_tiles = (a.N / a.bn - a.nb_full) * ((a.M + a.bm - 1) / a.bm);
-        fold = a.lora_words && !a.swiglu && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
+        fold = a.lora_words && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
                a.counters && row_tiles <= kPrefillFoldMaxTiles && row_tiles <= kProjectFoldCounters &&
                sliced_tiles <= kProjectFoldCounters && a.n_adapters >= 1 && a.n_adapters <= 8 && a.lora_a && a.lora_t &&
                a.ranks && a.scales && a.r_total <= kProjectMaxRank;
@@ -1045,7 +1048,6 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         }
     }
     if (a.bn != 128 && a.bn != 256) return hipErrorInvalidValue;
-    if (a.swiglu && a.r_total > 0) return hipErrorInvalidValue;  // the LoRA term has no gate/up split
     const int m_blocks = (a.M + a.bm - 1) / a.bm;
     const int KS = a.KS < 1 ? 1 : a.KS;
     const int GSb = (G + KS - 1) / KS;
@@ -1059,6 +1061,11 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     const int grid = prefill_grid(a.M, a.N, shape);
     if (fold) {
         pf.consumers = grid;
+        if (a.swiglu) {
+            if (a.bm == 128) return launch_shape_as<4, 1, 4, true, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
+            return rs ? launch_shape_as<4, 1, 2, true, true, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf)
+                      : launch_shape_as<4, 1, 2, true, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
+        }
         if (a.bm == 128) return launch_shape_as<4, 1, 4, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);
         return rs ? launch_shape_as<4, 1, 2, false, true, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf)
                   : launch_shape_as<4, 1, 2, false, false, true>(a, grid, m_blocks, RP, KS, GSb, max_groups, stream, pf);

@@ -29,7 +29,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 from . import marlin_gemm, marlin_proj
-from .lora import proj_forward
+from .lora import proj_forward, swiglu_forward, swiglu_lora_fits
 from .marlin_proj import MarlinPackedProj, MarlinProjError
 
 
@@ -88,16 +88,14 @@ class LayerProjections:
             y = y + ((x @ lora.a.t().to(x.dtype)) @ lora.b.t().to(x.dtype)) * lora_scale
         return y
 
-    def swiglu(self, x: torch.Tensor) -> torch.Tensor:
-        """`silu(gate_proj(x)) * up_proj(x)` (forward.rs:2771-2819): one fused launch on the
-        interleaved pack when it is installed, otherwise two projections and the elementwise ops."""
-        if self.gate_up_fused is not None:
-            w = self.gate_up_fused
-            x2 = x.reshape(-1, w.k).contiguous()
-            h = marlin_gemm.marlin_w4a16_gemm_swiglu(x2, w.b_packed, w.scales, w.groupsize)
-            return h.reshape(*x.shape[:-1], w.n // 2)
-        gate = self.forward(PackKind.GateProj, x)
-        up = self.forward(PackKind.UpProj, x)
+    def swiglu(self, x: torch.Tensor, gate_lora=None, up_lora=None, lora_scale: float = 1.0) -> torch.Tensor:
+        """`silu(gate_proj(x)) * up_proj(x)`, each projection with its LoRA delta (forward.rs:2771-2819):
+        one fused launch on the interleaved pack when it is installed and the adapters fit it (stacked
+        rank <= 64), otherwise two projections and the elementwise ops."""
+        if self.gate_up_fused is not None and swiglu_lora_fits(gate_lora, up_lora):
+            return swiglu_forward(x, self.gate_up_fused, gate_lora, up_lora, lora_scale)
+        gate = self.forward(PackKind.GateProj, x, gate_lora, lora_scale)
+        up = self.forward(PackKind.UpProj, x, up_lora, lora_scale)
         return torch.nn.functional.silu(gate) * up
 
 

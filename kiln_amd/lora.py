@@ -68,5 +68,47 @@ def proj_forward(x: torch.Tensor, packed: MarlinPackedProj, lora, lora_scale: fl
     return y2.reshape(*x.shape[:-1], packed.n)
 
 
+def _as_stacked(lora, lora_scale: float) -> Optional[StackedLora]:
+    if lora is None or isinstance(lora, StackedLora):
+        return lora
+    return stack_adapters([lora], [lora_scale])
+
+
+def swiglu_forward(x: torch.Tensor, gate_up: MarlinPackedProj, gate_lora=None, up_lora=None,
+                   lora_scale: float = 1.0) -> torch.Tensor:
+    """`silu(gate_proj(x) + d_gate) * (up_proj(x) + d_up)` on the interleaved gate/up pack in one launch:
+    the two `mlp_proj_forward` calls with `lora_layer.gate_proj` / `up_proj`, `silu` and the multiply of
+    forward.rs:2771-2819.  `gate_lora` / `up_lora` are None, a LoraProjectionWeights (scaled by
+    `lora_scale`) or a StackedLora; together at most 64 rank columns and 8 adapters."""
+    if x.dim() not in (2, 3) or x.shape[-1] != gate_up.k:
+        raise MarlinProjError(f"marlin_proj: x last-dim {x.shape[-1]} != packed weight k {gate_up.k}")
+    n_out = gate_up.n // 2
+    x2 = x.reshape(-1, gate_up.k).contiguous()
+    g, u = _as_stacked(gate_lora, lora_scale), _as_stacked(up_lora, lora_scale)
+    if g is None and u is None:
+        h = marlin_gemm.marlin_w4a16_gemm_swiglu(x2, gate_up.b_packed, gate_up.scales, gate_up.groupsize)
+        return h.reshape(*x.shape[:-1], n_out)
+    sides = [s for s in (g, u) if s is not None]
+    a_cat = torch.cat([s.a_cat for s in sides], dim=0).contiguous()
+    b_cat = marlin_gemm.interleave_gate_up_lora_b(g.b_cat if g is not None else None,
+                                                  u.b_cat if u is not None else None, n_out)
+    ranks = tuple(r for s in sides for r in s.ranks)
+    scales = tuple(v for s in sides for v in s.scales)
+    h = marlin_gemm.marlin_w4a16_gemm_swiglu_lora(x2, gate_up.b_packed, gate_up.scales, gate_up.groupsize,
+                                                  a_cat, b_cat, ranks, scales)
+    return h.reshape(*x.shape[:-1], n_out)
+
+
+def swiglu_lora_fits(gate_lora, up_lora) -> bool:
+    """Can `swiglu_forward` take these adapters (stacked rank <= 64, <= 8 adapters)?"""
+    ranks = []
+    for side in (gate_lora, up_lora):
+        if isinstance(side, StackedLora):
+            ranks += list(side.ranks)
+        elif side is not None:
+            ranks.append(int(side.a.shape[0]))
+    return sum(ranks) <= 64 and len(ranks) <= 8
+
+
 mlp_proj_forward = proj_forward
 q_proj_forward = proj_forward

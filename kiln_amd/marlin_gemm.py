@@ -296,3 +296,76 @@ def marlin_w4a16_gemm_lora(a: torch.Tensor, b_packed: torch.Tensor, scales: torc
         raise MarlinGemmError(f"kiln_w4a16_gemm_lora failed with status {status}: "
                               f"{_lib.status_string(status)} (m={m}, n={n}, k={k}, r_total={r_total})")
     return out
+
+
+def interleave_gate_up_lora_b(gate_b: torch.Tensor | None, up_b: torch.Tensor | None, n_out: int) -> torch.Tensor:
+    """The stacked `lora_b` `marlin_w4a16_gemm_swiglu_lora` reads, from gate's `[n_out, r_gate]` and up's
+    `[n_out, r_up]` column-concatenated B matrices (either may be None: no adapter on that projection):
+    `[2 n_out, r_gate + r_up]`, rows in the packed column order of `pack.interleave_gate_up` (per 16
+    rows 8 gate columns, then the 8 matching up columns); a gate row is `[B_gate row | 0]`, an up row
+    `[0 | B_up row]`."""
+    ref = gate_b if gate_b is not None else up_b
+    if ref is None:
+        _bail("at least one of gate's and up's LoRA B matrices is needed")
+    if n_out % 8 != 0:
+        _bail(f"n_out {n_out} must be a multiple of 8")
+    r_gate = 0 if gate_b is None else gate_b.shape[1]
+    r_up = 0 if up_b is None else up_b.shape[1]
+    for b in (gate_b, up_b):
+        if b is not None and (b.dim() != 2 or b.shape[0] != n_out or b.dtype != torch.bfloat16):
+            _bail(f"LoRA B matrices must be bf16 [n_out={n_out}, rank]")
+    out = torch.zeros((n_out // 8, 2, 8, r_gate + r_up), dtype=torch.bfloat16, device=ref.device)
+    if gate_b is not None:
+        out[:, 0, :, :r_gate] = gate_b.reshape(n_out // 8, 8, r_gate)
+    if up_b is not None:
+        out[:, 1, :, r_gate:] = up_b.reshape(n_out // 8, 8, r_up)
+    return out.reshape(2 * n_out, r_gate + r_up)
+
+
+def marlin_w4a16_gemm_swiglu_lora(a: torch.Tensor, b_packed: torch.Tensor, scales: torch.Tensor, groupsize: int,
+                                  lora_a: torch.Tensor, lora_b: torch.Tensor, ranks, lora_scales,
+                                  *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """`silu(gate + d_gate) * (up + d_up)`: `marlin_w4a16_gemm_swiglu` with LoRA adapters on gate_proj and
+    up_proj, the deltas added to the f32 sums before the product is formed and rounded once.
+
+    Fused form of the two `mlp_proj_forward` calls with `lora_layer.gate_proj` / `up_proj`, `silu` and the
+    multiply (crates/kiln-model/src/forward.rs:2771-2819).  `lora_a` is `[r_total, k]` (gate's adapters,
+    then up's, stacked along rows), `lora_b` `[2 n_out, r_total]` from `interleave_gate_up_lora_b`;
+    `ranks` / `lora_scales` one entry per stacked adapter.
+    """
+    m, k, n = _check_gemm_args(a, b_packed, scales, groupsize)
+    if n % 256 != 0:
+        _bail(f"fused gate+up width {n} must be a multiple of 256")
+    n_out = n // 2
+    ranks = [int(r) for r in ranks]
+    lora_scales = [float(v) for v in lora_scales]
+    r_total = sum(ranks)
+    if len(ranks) != len(lora_scales) or not ranks:
+        _bail("ranks and lora_scales must be non-empty and of equal length")
+    if tuple(lora_a.shape) != (r_total, k) or tuple(lora_b.shape) != (n, r_total):
+        _bail(f"LoRA shapes {tuple(lora_a.shape)} / {tuple(lora_b.shape)} do not match "
+              f"[r_total={r_total}, k={k}] / [2 n_out={n}, r_total={r_total}]")
+    if lora_a.dtype != torch.bfloat16 or lora_b.dtype != torch.bfloat16:
+        _bail("LoRA matrices must be bf16")
+    if not (lora_a.is_cuda and lora_b.is_cuda):
+        _bail("LoRA matrices must be on CUDA")
+    lib = _lib.load()
+    a, b_packed, scales = a.contiguous(), b_packed.contiguous(), scales.contiguous()
+    lora_a, lora_b = lora_a.contiguous(), lora_b.contiguous()
+    if out is None:
+        out = torch.empty((m, n_out), dtype=torch.bfloat16, device=a.device)
+    if m == 0:
+        return out
+    c_ranks = (ctypes.c_int * len(ranks))(*ranks)
+    c_scales = (ctypes.c_float * len(ranks))(*lora_scales)
+    with torch.cuda.device(a.device):
+        stream = torch.cuda.current_stream(a.device).cuda_stream
+        ws = _workspace(a.device, stream, lib.kiln_w4a16_swiglu_workspace_bytes(m, n_out, k))
+        status = lib.kiln_w4a16_gemm_swiglu_lora(
+            a.data_ptr(), b_packed.data_ptr(), out.data_ptr(), scales.data_ptr(), m, n_out, k,
+            ws.data_ptr(), groupsize, a.device.index or 0, stream, lora_a.data_ptr(),
+            lora_b.data_ptr(), r_total, len(ranks), c_ranks, c_scales)
+    if status != 0:
+        raise MarlinGemmError(f"kiln_w4a16_gemm_swiglu_lora failed with status {status}: "
+                              f"{_lib.status_string(status)} (m={m}, n_out={n_out}, k={k}, r_total={r_total})")
+    return out

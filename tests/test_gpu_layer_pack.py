@@ -98,3 +98,41 @@ def test_fused_gate_up_swiglu_of_a_layer(oracle, packed_layers):
         sides.append(oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128))
     err, _, _ = row_errors(bf16_bits(h), oracle.c_swiglu_f32(sides[0], sides[1]), oracle)
     assert tuple(h.shape) == (m, 9216) and err.max() <= 1e-2
+
+
+def test_fused_gate_up_swiglu_of_a_layer_with_adapters(oracle, packed_layers):
+    """`LayerProjections.swiglu` with a LoRA adapter on gate_proj and two stacked ones on up_proj: the
+    fused launch against the oracle's two projections + deltas + silu * up, and against the layer's
+    own unfused route (adapters too large for the fused entry point fall back to it)."""
+    from kiln_amd.lora import LoraProjectionWeights, stack_adapters
+    layers, host, _ = packed_layers
+    m = 24
+    x = oracle.gen_normal_bf16(m, HIDDEN, 1.0, 13)
+    adapters = {}
+    for name, ranks in (("gate", (16,)), ("up", (8, 16))):
+        adapters[name] = [(oracle.gen_normal_bf16(r, HIDDEN, 0.05, 40 + 7 * i + len(name)),
+                           oracle.gen_normal_bf16(9216, r, 0.05, 50 + 7 * i + len(name))) for i, r in enumerate(ranks)]
+    scales = {"gate": (0.5,), "up": (1.0, 2.0)}
+    sides = []
+    for kind, name in ((PackKind.GateProj, "gate"), (PackKind.UpProj, "up")):
+        codes, s_bits, _ = oracle.c_quantize(host[1][kind], 128)
+        y = oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128)
+        for (a_i, b_i), sc in zip(adapters[name], scales[name]):
+            oracle.c_lora_delta_add(y, x, a_i, b_i, sc)
+        sides.append(y)
+    h_ref = oracle.c_swiglu_f32(sides[0], sides[1])
+    stacked = {name: stack_adapters([LoraProjectionWeights(bf16_tensor(a_i), bf16_tensor(b_i)) for a_i, b_i in adapters[name]],
+                                    scales[name]) for name in adapters}
+    h = layers[1].swiglu(bf16_tensor(x), stacked["gate"], stacked["up"])
+    err, _, _ = row_errors(bf16_bits(h), h_ref, oracle)
+    assert tuple(h.shape) == (m, 9216) and err.max() <= 1e-2
+    # a single adapter given as LoraProjectionWeights with the call's scale, on gate only
+    a0, b0 = adapters["gate"][0]
+    h1 = layers[1].swiglu(bf16_tensor(x), LoraProjectionWeights(bf16_tensor(a0), bf16_tensor(b0)), None, 0.5)
+    codes, s_bits, _ = oracle.c_quantize(host[1][PackKind.UpProj], 128)
+    up_plain = oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128)
+    codes, s_bits, _ = oracle.c_quantize(host[1][PackKind.GateProj], 128)
+    gate1 = oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128)
+    oracle.c_lora_delta_add(gate1, x, a0, b0, 0.5)
+    err1, _, _ = row_errors(bf16_bits(h1), oracle.c_swiglu_f32(gate1, up_plain), oracle)
+    assert err1.max() <= 1e-2

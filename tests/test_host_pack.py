@@ -308,6 +308,27 @@ def test_interleave_gate_up_is_a_column_permutation(oracle):
                                 packs[1][0][:, :2 * 192].copy(), packs[1][1][:, :192].copy(), g)
 
 
+def test_interleave_gate_up_lora_b_follows_the_packed_columns():
+    """Rows of the stacked LoRA B in the column order of the interleaved pack (per 16 rows 8 gate
+    columns, then the 8 matching up columns), gate's entries in gate's rank columns, up's in up's."""
+    import torch
+    n_out, rg, ru = 32, 3, 5
+    gate = (torch.arange(n_out * rg, dtype=torch.float32).reshape(n_out, rg) + 1).to(torch.bfloat16)
+    up = -(torch.arange(n_out * ru, dtype=torch.float32).reshape(n_out, ru) + 1).to(torch.bfloat16)
+    out = marlin_gemm.interleave_gate_up_lora_b(gate, up, n_out)
+    assert tuple(out.shape) == (2 * n_out, rg + ru) and out.dtype == torch.bfloat16
+    for j in range(n_out // 8):
+        assert torch.equal(out[16 * j:16 * j + 8, :rg], gate[8 * j:8 * j + 8])
+        assert torch.equal(out[16 * j + 8:16 * j + 16, rg:], up[8 * j:8 * j + 8])
+        assert not out[16 * j:16 * j + 8, rg:].any() and not out[16 * j + 8:16 * j + 16, :rg].any()
+    only_up = marlin_gemm.interleave_gate_up_lora_b(None, up, n_out)
+    assert tuple(only_up.shape) == (2 * n_out, ru) and not only_up[0:8].any() and torch.equal(only_up[8:16], up[0:8])
+    with pytest.raises(marlin_gemm.MarlinGemmError):
+        marlin_gemm.interleave_gate_up_lora_b(None, None, n_out)
+    with pytest.raises(marlin_gemm.MarlinGemmError):
+        marlin_gemm.interleave_gate_up_lora_b(gate[:16], up, n_out)
+
+
 def test_bench_refuses_more_than_one_gpu():
     """bench.py measures one GPU only: --gpus 2 (or a multi-rank environment) exits with a message."""
     import os
