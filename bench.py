@@ -101,7 +101,10 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
     del sweep_w
 
     # fused gate+up + SwiGLU epilogue against the plain GEMM of the same packed width
-    from kiln_amd.marlin_gemm import marlin_w4a16_gemm_swiglu
+    from kiln_amd.marlin_gemm import marlin_w4a16_gemm_swiglu, marlin_w4a16_gemm_swiglu_lora
+    sl_ranks, sl_scales = (16, 16, 16, 16), (1.0, 1.0, 1.0, 1.0)   # two adapters on gate_proj, two on up_proj
+    sl_a = (torch.randn(sum(sl_ranks), 2560, device=dev) * 0.02).to(torch.bfloat16)
+    sl_b = (torch.randn(18432, sum(sl_ranks), device=dev) * 0.02).to(torch.bfloat16)
     for m_sg, count in ((16, 200), (2048, 72)):
         ws_ = [make_layer(2560, 18432) for _ in range(12)]
         x_ = torch.randn(m_sg, 2560, device=dev).to(torch.bfloat16)
@@ -115,10 +118,15 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
             marlin_gemm.marlin_w4a16_gemm(x_, b_, s_, GROUP, out=p_)
         # the plain GEMM on the same weights right next to it: at this point of the run (after the heavy
         # configurations) both read slower than the headline figure taken at the start
+        def fn_lora(i):
+            b_, s_ = ws_[i % 12]
+            marlin_w4a16_gemm_swiglu_lora(x_, b_, s_, GROUP, sl_a, sl_b, sl_ranks, sl_scales, out=o_)
         t_plain, _ = timed_graph(fn_plain, count)
         t, _ = timed_graph(fn, count)
+        t_lora, _ = timed_graph(fn_lora, count)
         extra[f"swiglu_m{m_sg}_gate_up"] = {"us": round(t / count * 1e6, 2),
-                                            "plain_gemm_same_weights_us": round(t_plain / count * 1e6, 2)}
+                                            "plain_gemm_same_weights_us": round(t_plain / count * 1e6, 2),
+                                            "with_two_lora_adapters_a_side_us": round(t_lora / count * 1e6, 2)}
 
     # per-launch distribution and wrapper-inclusive cost of the headline GEMM (eager launches)
     ws_ = [make_layer(2560, 18432) for _ in range(16)]
