@@ -44,7 +44,7 @@ def test_fused_lora_matches_oracle(oracle, m, k, n, ranks, scales):
 
 
 @pytest.mark.parametrize("k,n", [(2560, 18432), (9216, 2560), (2560, 8192)])
-@pytest.mark.parametrize("m", [1, 3, 16, 17, 32, 33, 48, 64, 80])
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 32, 33, 48, 64, 80, 128, 160])
 def test_lora_on_few_rows(oracle, m, k, n):
     """Few rows take the small-M kernels, which add the low-rank term where they store a tile (the
     decode kernel up to 16 rows, the mid-M kernel beyond); adapters large enough that a missing term fails."""
@@ -232,6 +232,9 @@ def test_adapters_with_zero_b_equal_the_plain_call_bit_for_bit(m, k, n):
     (48, 9216, 2560),      # ... K slices of the product and of the projection
     (17, 4096, 2560),      # ... which calls with adapters take from 17 rows on
     (24, 2560, 18432),
+    (128, 2560, 18432),    # ... a launch of more blocks than the chip holds at once: the producers still come first
+    (192, 2560, 8192),     # ... three runs of 64 rows
+    (96, 9216, 2560),
 ])
 def test_projection_inside_the_matrix_core_launch(m, k, n):
     """Beyond 16 rows the projection (on the matrix-core path also the row sums, where they come from a
