@@ -42,6 +42,8 @@ out.update({"pf_x_bf16": x, "pf_gate_qweight": q_gate, "pf_gate_scales_f16": s_g
             "pf_up_qweight": q_up, "pf_up_scales_f16": s_up,
             "pf_gate_y_f32": y_gate, "pf_up_y_f32": y_up,
             "pf_lora_a4": lora_a[0], "pf_lora_a8": lora_a[1], "pf_lora_b4": lora_b[0], "pf_lora_b8": lora_b[1],
-            "pf_lora_y_f32": y_lora, "pf_swiglu_h_f32": ref.c_swiglu_f32(y_gate, y_up)})
+            "pf_lora_y_f32": y_lora, "pf_swiglu_h_f32": ref.c_swiglu_f32(y_gate, y_up),
+            # silu(gate + its two adapters' deltas) * up: the fused gate+up call with adapters on gate_proj
+            "pf_swiglu_lora_h_f32": ref.c_swiglu_f32(y_lora, y_up)})
 np.savez_compressed(Path(__file__).with_name("w4a16_small.npz"), **out)
 print({k_: v.shape for k_, v in out.items()})

@@ -62,6 +62,7 @@ def test_oracle_reproduces_golden_fused_paths(oracle):
     for a_i, b_i, sc in ((G["pf_lora_a4"], G["pf_lora_b4"], 0.5), (G["pf_lora_a8"], G["pf_lora_b8"], 2.0)):
         oracle.c_lora_delta_add(y, x, a_i, b_i, sc)
     assert np.array_equal(y.view(np.uint32), G["pf_lora_y_f32"].view(np.uint32))
+    assert np.array_equal(oracle.c_swiglu_f32(y, up).view(np.uint32), G["pf_swiglu_lora_h_f32"].view(np.uint32))
 
 
 @pytest.mark.gpu
@@ -90,4 +91,10 @@ def test_gpu_matches_golden_fused_paths(oracle, matrix_core_kernel_from_33_rows)
     h = marlin_gemm.marlin_w4a16_gemm_swiglu(xt, bgt, sgt, g)
     torch.cuda.synchronize()
     err, _, _ = row_errors(bf16_bits(h), G["pf_swiglu_h_f32"], oracle)
+    assert err.max() <= 1e-2
+    # the same fused call with the two adapters on gate_proj (none on up_proj)
+    b_il = marlin_gemm.interleave_gate_up_lora_b(b_cat, None, 256)
+    hl = marlin_gemm.marlin_w4a16_gemm_swiglu_lora(xt, bgt, sgt, g, a_cat, b_il, [4, 8], [0.5, 2.0])
+    torch.cuda.synchronize()
+    err, _, _ = row_errors(bf16_bits(hl), G["pf_swiglu_lora_h_f32"], oracle)
     assert err.max() <= 1e-2
