@@ -33,6 +33,7 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_BF16_PEAK_TFLOPS = 2500.0
 GROUP = 128
 LAYERS = 16
+TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median replay is reported
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
 # copy (x1.9989 and x1.0): 12278.6 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
@@ -284,8 +285,13 @@ def main() -> int:
 
     stream = torch.cuda.Stream()
 
-    def timed_graph(fn, count):
-        """Capture `count` calls of fn(i) into one graph; replay once untimed, once timed."""
+    replay_log = {}
+
+    def timed_graph(fn, count, tag=None):
+        """Capture `count` calls of fn(i) into one graph; replay once untimed, then TIMED_REPLAYS times,
+        each replay timed on its own between two synchronisations (HIP events on the launch stream around
+        exactly `count` calls); returns the median replay (replay to replay the same graph reads +-3 %,
+        the first ones after a change of workload high)."""
         g = torch.cuda.CUDAGraph()
         with torch.cuda.stream(stream):
             for i in range(min(count, LAYERS)):
@@ -296,19 +302,24 @@ def main() -> int:
                     fn(i)
             g.replay()
             stream.synchronize()
-            e0 = torch.cuda.Event(enable_timing=True)
-            e1 = torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            e0.record(stream)
-            g.replay()
-            e1.record(stream)
-            torch.cuda.synchronize()
-            wall = time.perf_counter() - t0
-        return e0.elapsed_time(e1) * 1e-3, wall
+            runs = []
+            for _ in range(TIMED_REPLAYS):
+                e0 = torch.cuda.Event(enable_timing=True)
+                e1 = torch.cuda.Event(enable_timing=True)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                e0.record(stream)
+                g.replay()
+                e1.record(stream)
+                torch.cuda.synchronize()
+                runs.append((e0.elapsed_time(e1) * 1e-3, time.perf_counter() - t0))
+        runs.sort()
+        if tag:
+            replay_log[tag] = [round(t / count * 1e6, 3) for t, _ in runs]
+        return runs[len(runs) // 2]
 
-    t_step, wall_step = timed_graph(step, args.steps)
-    t_gu, _ = timed_graph(lambda i: run("gate_up", i), args.steps)
+    t_step, wall_step = timed_graph(step, args.steps, tag="step_us_per_replay_sorted")
+    t_gu, _ = timed_graph(lambda i: run("gate_up", i), args.steps, tag="m16_gate_up_us_per_replay_sorted")
     t_dn, _ = timed_graph(lambda i: run("down", i), args.steps)
 
     bytes_gu = algorithmic_bytes(M, *shapes["gate_up"])
@@ -408,13 +419,14 @@ def main() -> int:
                                "int4 group-128 weights, fp16 scales, bf16 activations",
                    "m": M, "groupsize": GROUP, "layers_rotated": LAYERS,
                    "algorithmic_bytes_per_step": bytes_step, "launch": "one HIP graph of all timed steps",
+                   "timed_replays": TIMED_REPLAYS, "statistic": "median replay",
                    "wall_ms_per_step": round(wall_step / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_M16_TRAFFIC_BYTES,
                      "kernel": "w4a16_decode_gmp_kernel<5, 2, 4, false> (gate+up, M=16, K=2560, N=18432)",
                      "us_per_launch": round(us_gu, 3), "algorithmic_bytes_per_launch": bytes_gu},
         "cpu_baseline": cpu_baseline,
-        "extra": extra,
+        "extra": {**extra, **replay_log},
     }
     print(json.dumps(result))
     return 0
