@@ -40,8 +40,11 @@ int kiln_marlin_proj_env_enabled(void);
 int kiln_marlin_proj_parallel_pack_disabled(void);
 
 /*
- * pack_from_bf16 (marlin_proj.rs:198-207): download a bf16 [k, n] row-major
- * weight from device `dev`, quantise and pack it on the host, upload.
+ * pack_from_bf16 (marlin_proj.rs:198-207): quantise and pack a bf16 [k, n] row-major
+ * weight that lies on device `dev`.  The reference downloads it, packs on the host and
+ * uploads; here two kernels do it where the weight lies (kiln_w4a16_quantize_and_pack_device,
+ * the same bits; they run on the device's default stream and the call returns when they are
+ * done).  KILN_W4A16_HOST_PACK in {1, true, yes} takes the reference's three-phase host route.
  * `dev` < 0 means "not on a GPU": skipped, as the reference does for non-CUDA
  * tensors (marlin_proj.rs:88-91).  *out is NULL unless the result is KILN_PROJ_OK.
  */
@@ -49,9 +52,10 @@ int kiln_marlin_proj_pack_from_bf16(const void *weight_t, int64_t k, int64_t n, 
                                     kiln_marlin_packed_proj_t **out);
 
 /*
- * pack_from_bf16_batch (marlin_proj.rs:230-262): serial downloads, the host
- * pack of all jobs in parallel (sequential under KILN_DISABLE_PARALLEL_PACK),
- * serial uploads.  outs[i] is NULL for skipped entries; order is preserved.
+ * pack_from_bf16_batch (marlin_proj.rs:230-262): every weight packed on the device in
+ * turn; on the host route (KILN_W4A16_HOST_PACK) serial downloads, the host pack of all jobs
+ * in parallel (sequential under KILN_DISABLE_PARALLEL_PACK), serial uploads.
+ * outs[i] is NULL for skipped entries; order is preserved.
  */
 int kiln_marlin_proj_pack_from_bf16_batch(const void *const *weights_t, const int64_t *ks, const int64_t *ns,
                                           const int *groupsizes, int count, int dev,

@@ -186,6 +186,17 @@ kiln_marlin_status_t kiln_w4a16_dequant_f32(
     const void *B, const void *s, int prob_k, int prob_n, int groupsize,
     void *out, int dev, void *stream);
 
+/*
+ * Quantise a bf16 [k, n] weight that is already in device memory and pack it there: the same
+ * quantiser as kiln_w4a16_quantize_and_pack below (lib.rs:393-427) and the same bits out, without
+ * the download, host pack and upload of crates/kiln-model/src/marlin_proj.rs:86-181 (the reference
+ * has no device-side counterpart; its host pack costs 17-58 s per model load).  b_packed: k*n/8
+ * int32, scales_f16: (k/g)*n fp16, both device memory; the two kernels run on `stream`.
+ */
+kiln_marlin_status_t kiln_w4a16_quantize_and_pack_device(
+    const void *weight_bf16, int k, int n, int groupsize,
+    void *b_packed, void *scales_f16, int dev, void *stream);
+
 /* ---- host-side packing (pure CPU, thread-safe, no GPU state) ------------ */
 
 /*

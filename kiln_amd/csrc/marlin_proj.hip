@@ -152,10 +152,48 @@ int upload_packed(const PackedHost &packed, int dev, kiln_marlin_packed_proj_t *
     return KILN_PROJ_OK;
 }
 
+// The three phases in one: the weight is quantised and packed where it lies, by two kernels on the
+// device's default stream (same bits as the host quantiser; KILN_W4A16_HOST_PACK=1 keeps the host
+// route of marlin_proj.rs:86-181).  Same validation, same results and messages as prepare_pack_job.
+int pack_on_device(const void *weight_t, int64_t k, int64_t n, int groupsize, int dev,
+                   kiln_marlin_packed_proj_t **out) {
+    *out = nullptr;
+    if (dev < 0) return KILN_PROJ_SKIPPED;
+    if (!weight_t) return fail("marlin_proj: weight_t must be a 2D [k, n] tensor");
+    if (!shape_is_supported(k, n)) return KILN_PROJ_SKIPPED;
+    if (!(groupsize == -1 || groupsize == 128))
+        return fail("marlin_proj: groupsize must be -1 or 128 (got " + std::to_string(groupsize) + ")");
+    if (k > INT32_MAX || n > INT32_MAX) return fail("marlin_proj: weight too large");
+    DeviceScope scope(dev);
+    if (!scope.ok) return fail("marlin_proj: pack on device");
+    auto w = std::make_unique<kiln_marlin_packed_proj>();
+    w->k = k;
+    w->n = n;
+    w->groupsize = groupsize;
+    w->dev = dev;
+    const size_t b_bytes = (size_t)k * n / 8 * sizeof(int32_t);
+    const size_t s_bytes = num_groups(k, groupsize) * (size_t)n * sizeof(uint16_t);
+    if (hipMalloc(&w->b_packed, b_bytes) != hipSuccess) return fail("marlin_proj: allocate b_packed on device");
+    if (hipMalloc(&w->scales, s_bytes) != hipSuccess) {
+        (void)hipFree(w->b_packed);
+        return fail("marlin_proj: allocate scales on device");
+    }
+    const int st = kiln_w4a16_quantize_and_pack_device(weight_t, (int)k, (int)n, groupsize, w->b_packed, w->scales, dev,
+                                                       nullptr);
+    if (st != KILN_W4A16_OK || hipStreamSynchronize(nullptr) != hipSuccess) {
+        (void)hipFree(w->b_packed);
+        (void)hipFree(w->scales);
+        return fail(std::string("marlin_proj: pack on device: ") + kiln_w4a16_status_string((kiln_marlin_status_t)st));
+    }
+    *out = w.release();
+    return KILN_PROJ_OK;
+}
+
 // marlin_proj.rs:198-207
 int pack_from_bf16(const void *weight_t, int64_t k, int64_t n, int groupsize, int dev,
                    kiln_marlin_packed_proj_t **out) {
     *out = nullptr;
+    if (!env_truthy("KILN_W4A16_HOST_PACK")) return pack_on_device(weight_t, k, n, groupsize, dev, out);
     std::optional<PackJobHost> job;
     const int st = prepare_pack_job(weight_t, k, n, groupsize, dev, job);
     if (st != KILN_PROJ_OK) return st;
@@ -167,6 +205,19 @@ int pack_from_bf16_batch(const void *const *weights_t, const int64_t *ks, const 
                          int count, int dev, kiln_marlin_packed_proj_t **outs) {
     for (int i = 0; i < count; ++i) outs[i] = nullptr;
     if (count <= 0) return KILN_PROJ_OK;
+    if (!env_truthy("KILN_W4A16_HOST_PACK")) {  // nothing to overlap: every weight is packed where it lies
+        for (int i = 0; i < count; ++i) {
+            const int st = pack_on_device(weights_t[i], ks[i], ns[i], groupsizes[i], dev, &outs[i]);
+            if (st == KILN_PROJ_ERR) {
+                for (int j = 0; j < i; ++j) {
+                    kiln_marlin_proj_free(outs[j]);
+                    outs[j] = nullptr;
+                }
+                return st;
+            }
+        }
+        return KILN_PROJ_OK;
+    }
     std::vector<std::optional<PackJobHost>> jobs((size_t)count);
     for (int i = 0; i < count; ++i) {
         const int st = prepare_pack_job(weights_t[i], ks[i], ns[i], groupsizes[i], dev, jobs[i]);

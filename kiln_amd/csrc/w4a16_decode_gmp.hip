@@ -177,7 +177,7 @@ struct GmpTailArgs {
 struct GmpParkedTail {
     uint32_t w[8];
 };
-__device__ __forceinline__ GmpParkedTail gmp_park(const GmpTailArgs &t) {
+[[maybe_unused]] __device__ __forceinline__ GmpParkedTail gmp_park(const GmpTailArgs &t) {
     struct Words {
         uint32_t w[8];
     } in = __builtin_bit_cast(Words, t);
@@ -186,7 +186,7 @@ __device__ __forceinline__ GmpParkedTail gmp_park(const GmpTailArgs &t) {
     for (int i = 0; i < 8; ++i) asm volatile("v_mov_b32 %0, %1" : "=v"(p.w[i]) : "s"(in.w[i]));
     return p;
 }
-__device__ __forceinline__ GmpTailArgs gmp_unpark(const GmpParkedTail &p) {
+[[maybe_unused]] __device__ __forceinline__ GmpTailArgs gmp_unpark(const GmpParkedTail &p) {
     struct Words {
         uint32_t w[8];
     } out;

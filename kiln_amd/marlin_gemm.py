@@ -164,6 +164,28 @@ def quantize_and_pack(weight, k: int, n: int, groupsize: int, want_dequant: bool
     return b_packed, scales, dequant
 
 
+def quantize_and_pack_device(weight_t: torch.Tensor, groupsize: int):
+    """`quantize_and_pack` for a bf16 `[k, n]` weight that is already on the GPU: the same quantiser
+    (lib.rs:393-427) run there, the same bits out -- `(b_packed int32 [k/16, 2n], scales f16 [k/g, n])`
+    as CUDA tensors -- without the download, host pack and upload of marlin_proj.rs:86-181."""
+    if weight_t.dim() != 2 or weight_t.dtype != torch.bfloat16 or not weight_t.is_cuda:
+        _bail("weight_t must be a 2D [k, n] bf16 CUDA tensor")
+    k, n = weight_t.shape
+    if k % 128 != 0 or n % 256 != 0 or not (groupsize == -1 or groupsize == 128):
+        _bail(f"unsupported shape k={k} n={n} groupsize={groupsize} (k % 128, n % 256, groupsize -1 or 128)")
+    weight_t = weight_t.contiguous()
+    g = k if groupsize == -1 else groupsize
+    b_packed = torch.empty((k // 16, 2 * n), dtype=torch.int32, device=weight_t.device)
+    scales = torch.empty((k // g, n), dtype=torch.float16, device=weight_t.device)
+    with torch.cuda.device(weight_t.device):
+        stream = torch.cuda.current_stream(weight_t.device).cuda_stream
+        st = _lib.load().kiln_w4a16_quantize_and_pack_device(weight_t.data_ptr(), k, n, groupsize, b_packed.data_ptr(),
+                                                             scales.data_ptr(), weight_t.device.index or 0, stream)
+    if st != 0:
+        raise MarlinGemmError(f"kiln_w4a16_quantize_and_pack_device: {_lib.status_string(st)}")
+    return b_packed, scales
+
+
 def repack_gptq(qweight, scales_f16, qzeros=None, groupsize: int = 128):
     """One-time repack of GPTQ-canonical tensors (`qweight [k/8, n]` int32, `scales [k/g, n]`
     f16, optional `qzeros [k/g, n/8]`; quantized.rs:1-14) into the tile layout."""
@@ -219,6 +241,7 @@ def interleave_gate_up(gate_b, gate_s, up_b, up_s, groupsize: int = 128):
 
 
 pack = SimpleNamespace(MAX_Q=MAX_Q, Q_OFFSET=Q_OFFSET, quantize_and_pack=quantize_and_pack,
+                       quantize_and_pack_device=quantize_and_pack_device,
                        repack_gptq=repack_gptq, unpack_to_gptq=unpack_to_gptq,
                        interleave_gate_up=interleave_gate_up)
 
