@@ -197,6 +197,14 @@ kiln_marlin_status_t kiln_w4a16_quantize_and_pack_device(
     const void *weight_bf16, int k, int n, int groupsize,
     void *b_packed, void *scales_f16, int dev, void *stream);
 
+/*
+ * kiln_w4a16_interleave_gate_up (below) for packed projections that are in device memory: one
+ * copy kernel on `stream`, same bits.  out_b: k * 2 n_each / 8 int32, out_s: (k/g) * 2 n_each fp16.
+ */
+kiln_marlin_status_t kiln_w4a16_interleave_gate_up_device(
+    const void *gate_b, const void *gate_s, const void *up_b, const void *up_s,
+    int k, int n_each, int groupsize, void *out_b, void *out_s, int dev, void *stream);
+
 /* ---- host-side packing (pure CPU, thread-safe, no GPU state) ------------ */
 
 /*

@@ -127,8 +127,46 @@ __global__ __launch_bounds__(256) void w4a16_pack_codes_kernel(const uint16_t *_
     b_packed[((size_t)nt * G + g) * (kChunkWords / 4) + lane] = u32x4{words[0], words[1], words[2], words[3]};
 }
 
+// Gate and up of equal shape into the pack the fused SwiGLU entry point reads (output tile j = gate
+// columns 8 j ... 8 j + 7, then the same up columns: kiln_w4a16_interleave_gate_up on the host).  One
+// wavefront per output chunk: lane c + 16 kq copies the 16 bytes of its source lane.
+__global__ __launch_bounds__(256) void w4a16_interleave_kernel(const u32x4 *__restrict__ gate_b,
+                                                               const uint16_t *__restrict__ gate_s,
+                                                               const u32x4 *__restrict__ up_b,
+                                                               const uint16_t *__restrict__ up_s, int G, int Gs,
+                                                               u32x4 *__restrict__ out_b, uint16_t *__restrict__ out_s) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int j = blockIdx.x * 4 + wave, g = blockIdx.y;
+    const int c = lane & 15, kq = lane >> 4;
+    const int src_tile = j >> 1, src_c = 8 * (j & 1) + (c & 7);
+    const bool up = (c & 8) != 0;
+    const u32x4 *src_b = up ? up_b : gate_b;
+    out_b[((size_t)j * G + g) * (kChunkWords / 4) + lane] = src_b[((size_t)src_tile * G + g) * (kChunkWords / 4) + src_c + 16 * kq];
+    if (g < Gs && kq == 0) {
+        const uint16_t *src_s = up ? up_s : gate_s;
+        out_s[((size_t)j * Gs + g) * kTileN + c] = src_s[((size_t)src_tile * Gs + g) * kTileN + src_c];
+    }
+}
+
 }  // namespace
 }  // namespace kiln
+
+extern "C" kiln_marlin_status_t kiln_w4a16_interleave_gate_up_device(const void *gate_b, const void *gate_s,
+                                                                     const void *up_b, const void *up_s, int k,
+                                                                     int n_each, int groupsize, void *out_b,
+                                                                     void *out_s, int dev, void *stream) {
+    using namespace kiln;
+    (void)dev;
+    if (!gate_b || !gate_s || !up_b || !up_s || !out_b || !out_s) return KILN_W4A16_ERR_ARGUMENT;
+    if (k <= 0 || k % 128 != 0 || n_each <= 0 || n_each % 128 != 0 || !(groupsize == -1 || groupsize == 128))
+        return KILN_W4A16_ERR_PROB_SHAPE;
+    const int G = k / kGroupK, Gs = groupsize == -1 ? 1 : G;
+    if (G > 65535) return KILN_W4A16_ERR_PROB_SHAPE;  // grid y
+    w4a16_interleave_kernel<<<dim3(n_each / 8 / 4, G), 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(
+        (const u32x4 *)gate_b, (const uint16_t *)gate_s, (const u32x4 *)up_b, (const uint16_t *)up_s, G, Gs,
+        (u32x4 *)out_b, (uint16_t *)out_s);
+    return hipGetLastError() == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+}
 
 extern "C" kiln_marlin_status_t kiln_w4a16_quantize_and_pack_device(const void *weight_bf16, int k, int n, int groupsize,
                                                                     void *b_packed, void *scales_f16, int dev,

@@ -146,10 +146,7 @@ def pack_layers(layers: Sequence[LayerProjections], kinds: Optional[Sequence[Pac
             g, u = layer.packed.get(PackKind.GateProj), layer.packed.get(PackKind.UpProj)
             if g is None or u is None or g.k != u.k or g.n != u.n or g.n % 128 != 0:
                 continue
-            b_gu, s_gu = marlin_gemm.interleave_gate_up(g.b_packed.cpu().numpy(), g.scales.cpu().numpy(),
-                                                        u.b_packed.cpu().numpy(), u.scales.cpu().numpy(), g.groupsize)
-            dev = g.b_packed.device
-            layer.gate_up_fused = MarlinPackedProj(torch.from_numpy(b_gu).to(dev), torch.from_numpy(s_gu).to(dev),
-                                                   g.groupsize, g.k, 2 * g.n)
+            b_gu, s_gu = marlin_gemm.interleave_gate_up_device(g.b_packed, g.scales, u.b_packed, u.scales, g.groupsize)
+            layer.gate_up_fused = MarlinPackedProj(b_gu, s_gu, g.groupsize, g.k, 2 * g.n)
             n_fused += 1
     return {"inputs": len(inputs), "packed": n_packed, "kept_bf16": len(inputs) - n_packed, "gate_up_fused": n_fused}

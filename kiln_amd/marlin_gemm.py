@@ -240,7 +240,31 @@ def interleave_gate_up(gate_b, gate_s, up_b, up_s, groupsize: int = 128):
     return out_b, out_s
 
 
+def interleave_gate_up_device(gate_b: torch.Tensor, gate_s: torch.Tensor, up_b: torch.Tensor, up_s: torch.Tensor,
+                              groupsize: int = 128):
+    """`interleave_gate_up` for packed projections that are CUDA tensors: one copy kernel, same bits."""
+    for t in (gate_b, gate_s, up_b, up_s):
+        if not t.is_cuda:
+            _bail("interleave_gate_up_device takes CUDA tensors")
+    if gate_b.shape != up_b.shape or gate_s.shape != up_s.shape or gate_b.dtype != torch.int32 or \
+            up_b.dtype != torch.int32 or gate_s.dtype != torch.float16 or up_s.dtype != torch.float16:
+        _bail("kiln-marlin-gemm: gate and up must have the same packed shapes (int32 words, fp16 scales)")
+    k, n_each = gate_b.shape[0] * 16, gate_b.shape[1] // 2
+    gate_b, gate_s, up_b, up_s = gate_b.contiguous(), gate_s.contiguous(), up_b.contiguous(), up_s.contiguous()
+    out_b = torch.empty((k // 16, 4 * n_each), dtype=torch.int32, device=gate_b.device)
+    out_s = torch.empty((gate_s.shape[0], 2 * n_each), dtype=torch.float16, device=gate_b.device)
+    with torch.cuda.device(gate_b.device):
+        stream = torch.cuda.current_stream(gate_b.device).cuda_stream
+        st = _lib.load().kiln_w4a16_interleave_gate_up_device(gate_b.data_ptr(), gate_s.data_ptr(), up_b.data_ptr(),
+                                                              up_s.data_ptr(), k, n_each, groupsize, out_b.data_ptr(),
+                                                              out_s.data_ptr(), gate_b.device.index or 0, stream)
+    if st != 0:
+        raise MarlinGemmError(f"kiln_w4a16_interleave_gate_up_device: {_lib.status_string(st)}")
+    return out_b, out_s
+
+
 pack = SimpleNamespace(MAX_Q=MAX_Q, Q_OFFSET=Q_OFFSET, quantize_and_pack=quantize_and_pack,
+                       interleave_gate_up_device=interleave_gate_up_device,
                        quantize_and_pack_device=quantize_and_pack_device,
                        repack_gptq=repack_gptq, unpack_to_gptq=unpack_to_gptq,
                        interleave_gate_up=interleave_gate_up)

@@ -61,3 +61,20 @@ def test_projection_layer_packs_on_the_device_with_the_host_routes_bits(oracle, 
     assert torch.equal(on_device.b_packed, on_host.b_packed) and torch.equal(on_device.scales, on_host.scales)
     x = bf16_tensor(oracle.gen_normal_bf16(4, k, 1.0, seed=4))
     assert torch.equal(marlin_proj.matmul_bf16(x, on_device), marlin_proj.matmul_bf16(x, on_host))
+
+
+@pytest.mark.parametrize("k,n_each,groupsize", [(256, 256, 128), (2560, 9216, 128), (512, 1280, -1)])
+def test_device_interleave_equals_host_interleave(oracle, k, n_each, groupsize):
+    """`kiln_w4a16_interleave_gate_up_device` against the host routine (which tests/test_host_pack.py
+    checks column by column): same words, same scales."""
+    sides = []
+    for seed in (1, 2):
+        codes = oracle.gen_codes(k, n_each, seed)
+        s_bits = oracle.gen_scales_f16(k, n_each, groupsize, seed)
+        sides.append(pack.repack_gptq(oracle.np_pack_gptq(codes), s_bits, None, groupsize))
+    b_host, s_host = pack.interleave_gate_up(sides[0][0], sides[0][1], sides[1][0], sides[1][1], groupsize)
+    dev = [(torch.from_numpy(np.asarray(b)).cuda(), torch.from_numpy(np.asarray(s).view(np.float16)).cuda()) for b, s in sides]
+    b_dev, s_dev = pack.interleave_gate_up_device(dev[0][0], dev[0][1], dev[1][0], dev[1][1], groupsize)
+    torch.cuda.synchronize()
+    assert np.array_equal(b_dev.cpu().numpy(), b_host)
+    assert np.array_equal(s_dev.cpu().numpy().view(np.uint16), np.asarray(s_host).view(np.uint16))
