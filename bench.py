@@ -165,6 +165,28 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
         host = (time.perf_counter() - t0) / n_calls * 1e6
         torch.cuda.synchronize()
     extra["m16_gate_up_c_entry_host_us_per_call"] = round(host, 2)
+
+    # quantise-and-pack of one layer's seven projections from bf16 weights in device memory (what a model load
+    # does 32 times): the device route, and the reference's download / host pack / upload route on 7 of them once
+    import os
+    from kiln_amd import marlin_proj
+    layer_shapes = [(2560, 8192), (2560, 1024), (2560, 1024), (4096, 2560), (2560, 9216), (2560, 9216), (9216, 2560)]
+    layer_w = [((torch.randn(k_, n_, device=dev) * 0.02).to(torch.bfloat16), GROUP) for k_, n_ in layer_shapes]
+    pack_ms = {}
+    for route in ("device", "device", "host"):
+        if route == "host":
+            os.environ["KILN_W4A16_HOST_PACK"] = "1"
+        try:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            packed = marlin_proj.pack_from_bf16_batch(layer_w)
+            torch.cuda.synchronize()
+            pack_ms[route] = round((time.perf_counter() - t0) * 1e3, 2)
+            del packed
+        finally:
+            os.environ.pop("KILN_W4A16_HOST_PACK", None)
+    extra["pack_one_layer_7_projections_ms"] = {"on_device": pack_ms["device"], "host_route": pack_ms["host"],
+                                                 "weights_millions": round(sum(k_ * n_ for k_, n_ in layer_shapes) / 1e6, 1)}
     return extra
 
 
@@ -177,7 +199,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the legs reported under `extra` (every launch is then an M=16 launch of the workload)")
-    ap.add_argument("--profile", choices=["decode", "decode_m1", "mid", "prefill", "lora"], default=None,
+    ap.add_argument("--profile", choices=["decode", "decode_m1", "mid", "prefill", "lora", "pack"], default=None,
                     help="for rocprofv3: launch K eager steps of the chosen regime (no graph, no CPU "
                          "baseline, no extra legs) plus one 64 MiB device copy that calibrates the "
                          "memory-traffic counters, print no JSON; decode_m1: gate+up, down and the "
@@ -252,6 +274,12 @@ def main() -> int:
                 for name in sweep:
                     b, s = layers[i % LAYERS][name] if name in shapes else sw[name][i % 8]
                     marlin_gemm.marlin_w4a16_gemm(x64[name], b, s, GROUP, out=o64[name])
+        elif args.profile == "pack":
+            from kiln_amd.marlin_gemm import pack as kpack
+            for name, kn in {"in_proj": (2560, 8192), "out_proj": (4096, 2560), **shapes}.items():
+                w_ = (torch.randn(*kn, device=dev) * 0.02).to(torch.bfloat16)
+                for i in range(args.steps):
+                    kpack.quantize_and_pack_device(w_, GROUP)
         elif args.profile == "lora":
             ranks, lscales = (16, 32), (0.5, 1.0)
             ad = {name: ((torch.randn(sum(ranks), kn[0], device=dev) * 0.02).to(torch.bfloat16),
