@@ -205,6 +205,15 @@ kiln_marlin_status_t kiln_w4a16_interleave_gate_up_device(
     const void *gate_b, const void *gate_s, const void *up_b, const void *up_s,
     int k, int n_each, int groupsize, void *out_b, void *out_s, int dev, void *stream);
 
+/*
+ * kiln_w4a16_repack_gptq (below) for GPTQ tensors that are in device memory: same bits, no
+ * re-quantisation.  With qzeros the call waits for `stream` once (the zero-points must all be 8
+ * before anything is written; not for use under graph capture); without, it only launches.
+ */
+kiln_marlin_status_t kiln_w4a16_repack_gptq_device(
+    const void *qweight, const void *scales_f16, const void *qzeros,
+    int k, int n, int groupsize, void *b_packed, void *scales_tiled, int dev, void *stream);
+
 /* ---- host-side packing (pure CPU, thread-safe, no GPU state) ------------ */
 
 /*

@@ -23,6 +23,7 @@ EXPORTS = (
     "kiln_w4a16_gemm_swiglu_lora",
     "kiln_w4a16_quantize_and_pack_device",
     "kiln_w4a16_interleave_gate_up_device",
+    "kiln_w4a16_repack_gptq_device",
     "kiln_w4a16_interleave_gate_up",
     "kiln_w4a16_dequant_f32",
     "kiln_w4a16_quantize_and_pack",
@@ -155,6 +156,8 @@ def _load(tuning: bool) -> ctypes.CDLL:
     L.kiln_w4a16_gemm_swiglu_lora.argtypes = L.kiln_w4a16_gemm_lora.argtypes
     L.kiln_w4a16_quantize_and_pack_device.restype = i
     L.kiln_w4a16_quantize_and_pack_device.argtypes = [vp, i, i, i, vp, vp, i, vp]
+    L.kiln_w4a16_repack_gptq_device.restype = i
+    L.kiln_w4a16_repack_gptq_device.argtypes = [vp, vp, vp, i, i, i, vp, vp, i, vp]
     L.kiln_w4a16_interleave_gate_up_device.restype = i
     L.kiln_w4a16_interleave_gate_up_device.argtypes = [vp, vp, vp, vp, i, i, i, vp, vp, i, vp]
     L.kiln_w4a16_swiglu_workspace_bytes.restype = c.c_size_t

@@ -148,8 +148,70 @@ __global__ __launch_bounds__(256) void w4a16_interleave_kernel(const u32x4 *__re
     }
 }
 
+// GPTQ-canonical tensors (qweight [k/8, n] int32 with row j of eight in bits 4 j, scales [k/g, n] fp16;
+// crates/kiln-model/src/quantized.rs:1-14, :127-152) into the tile layout: kiln_w4a16_repack_gptq on the
+// host.  One wavefront per chunk; lane c + 16 kq gathers its four source words and moves each nibble to
+// its place in the layout's word.  No re-quantisation: the codes are the checkpoint's.
+__device__ __forceinline__ uint32_t pack_shuffle_nibbles(uint32_t w) {
+    uint32_t out = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out |= ((w >> (4 * j)) & 0xFu) << (4 * nibble_pos(j));
+    return out;
+}
+
+__global__ __launch_bounds__(256) void w4a16_repack_gptq_kernel(const uint32_t *__restrict__ qweight,
+                                                                const uint16_t *__restrict__ scales, int n, int G, int Gs,
+                                                                u32x4 *__restrict__ b_packed,
+                                                                uint16_t *__restrict__ scales_tiled) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int nt = blockIdx.x * 4 + wave, g = blockIdx.y;
+    const int c = lane & 15, kq = lane >> 4;
+    const int col = nt * kTileN + c;
+    uint32_t words[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        words[t] = pack_shuffle_nibbles(qweight[(size_t)((g * kGroupK + 32 * t + 8 * kq) / 8) * n + col]);
+    b_packed[((size_t)nt * G + g) * (kChunkWords / 4) + lane] = u32x4{words[0], words[1], words[2], words[3]};
+    if (g < Gs && kq == 0) scales_tiled[scale_index(g, col, Gs)] = scales[(size_t)g * n + col];
+}
+
+// 1 in *bad if any packed zero-point word differs from 0x88888888 (zero-point 8 in all eight nibbles)
+__global__ void w4a16_check_qzeros_kernel(const uint32_t *__restrict__ qzeros, size_t count, int *bad) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        if (qzeros[i] != 0x88888888u) *bad = 1;
+}
+
 }  // namespace
 }  // namespace kiln
+
+extern "C" kiln_marlin_status_t kiln_w4a16_repack_gptq_device(const void *qweight, const void *scales, const void *qzeros,
+                                                              int k, int n, int groupsize, void *b_packed,
+                                                              void *scales_tiled, int dev, void *stream) {
+    using namespace kiln;
+    (void)dev;
+    if (!qweight || !scales || !b_packed || !scales_tiled) return KILN_W4A16_ERR_ARGUMENT;
+    if (k <= 0 || n <= 0 || k % 128 != 0 || n % 256 != 0 || !(groupsize == -1 || groupsize == 128))
+        return KILN_W4A16_ERR_PROB_SHAPE;
+    const int G = k / kGroupK, Gs = groupsize == -1 ? 1 : G;
+    if (G > 65535) return KILN_W4A16_ERR_PROB_SHAPE;  // grid y
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+    if (qzeros) {
+        // the zero-points must all be 8, as on the host route; the answer is needed before anything is written, so
+        // this one check waits for the stream.  The flag lives at the start of the output and is overwritten below.
+        int *flag = reinterpret_cast<int *>(b_packed);
+        int bad = 0;
+        if (hipMemsetAsync(flag, 0, sizeof(int), st) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
+        w4a16_check_qzeros_kernel<<<64, 256, 0, st>>>((const uint32_t *)qzeros, (size_t)Gs * (n / 8), flag);
+        if (hipGetLastError() != hipSuccess ||
+            hipMemcpyAsync(&bad, flag, sizeof(int), hipMemcpyDeviceToHost, st) != hipSuccess ||
+            hipStreamSynchronize(st) != hipSuccess)
+            return KILN_W4A16_ERR_LAUNCH;
+        if (bad) return KILN_W4A16_ERR_ZERO_POINT;
+    }
+    w4a16_repack_gptq_kernel<<<dim3(n / 64, G), 256, 0, st>>>((const uint32_t *)qweight, (const uint16_t *)scales, n, G, Gs,
+                                                               (u32x4 *)b_packed, (uint16_t *)scales_tiled);
+    return hipGetLastError() == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+}
 
 extern "C" kiln_marlin_status_t kiln_w4a16_interleave_gate_up_device(const void *gate_b, const void *gate_s,
                                                                      const void *up_b, const void *up_s, int k,

@@ -240,6 +240,32 @@ def interleave_gate_up(gate_b, gate_s, up_b, up_s, groupsize: int = 128):
     return out_b, out_s
 
 
+def repack_gptq_device(qweight: torch.Tensor, scales_f16: torch.Tensor, qzeros: torch.Tensor | None = None,
+                       groupsize: int = 128):
+    """`repack_gptq` for GPTQ tensors that are CUDA tensors (`qweight [k/8, n]` int32, `scales [k/g, n]` f16,
+    optional `qzeros [k/g, n/8]` int32): the same packed words and scales, formed on the GPU."""
+    if not (qweight.is_cuda and scales_f16.is_cuda) or qweight.dtype != torch.int32 or scales_f16.dtype != torch.float16:
+        _bail("repack_gptq_device takes CUDA tensors: int32 qweight, float16 scales")
+    k, n = qweight.shape[0] * 8, qweight.shape[1]
+    g = k if groupsize == -1 else groupsize
+    if tuple(scales_f16.shape) != (k // g, n):
+        _bail(f"scales must be [{k // g}, {n}]")
+    if qzeros is not None and (not qzeros.is_cuda or qzeros.dtype != torch.int32 or tuple(qzeros.shape) != (k // g, n // 8)):
+        _bail(f"qzeros must be a CUDA int32 [{k // g}, {n // 8}] tensor")
+    qweight, scales_f16 = qweight.contiguous(), scales_f16.contiguous()
+    qzeros = qzeros.contiguous() if qzeros is not None else None
+    b_packed = torch.empty((k // 16, 2 * n), dtype=torch.int32, device=qweight.device)
+    scales = torch.empty((k // g, n), dtype=torch.float16, device=qweight.device)
+    with torch.cuda.device(qweight.device):
+        stream = torch.cuda.current_stream(qweight.device).cuda_stream
+        st = _lib.load().kiln_w4a16_repack_gptq_device(qweight.data_ptr(), scales_f16.data_ptr(),
+                                                       qzeros.data_ptr() if qzeros is not None else None, k, n, groupsize,
+                                                       b_packed.data_ptr(), scales.data_ptr(), qweight.device.index or 0, stream)
+    if st != 0:
+        raise MarlinGemmError(f"kiln_w4a16_repack_gptq_device: {_lib.status_string(st)}")
+    return b_packed, scales
+
+
 def interleave_gate_up_device(gate_b: torch.Tensor, gate_s: torch.Tensor, up_b: torch.Tensor, up_s: torch.Tensor,
                               groupsize: int = 128):
     """`interleave_gate_up` for packed projections that are CUDA tensors: one copy kernel, same bits."""
@@ -264,7 +290,7 @@ def interleave_gate_up_device(gate_b: torch.Tensor, gate_s: torch.Tensor, up_b: 
 
 
 pack = SimpleNamespace(MAX_Q=MAX_Q, Q_OFFSET=Q_OFFSET, quantize_and_pack=quantize_and_pack,
-                       interleave_gate_up_device=interleave_gate_up_device,
+                       interleave_gate_up_device=interleave_gate_up_device, repack_gptq_device=repack_gptq_device,
                        quantize_and_pack_device=quantize_and_pack_device,
                        repack_gptq=repack_gptq, unpack_to_gptq=unpack_to_gptq,
                        interleave_gate_up=interleave_gate_up)

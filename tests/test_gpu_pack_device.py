@@ -78,3 +78,25 @@ def test_device_interleave_equals_host_interleave(oracle, k, n_each, groupsize):
     torch.cuda.synchronize()
     assert np.array_equal(b_dev.cpu().numpy(), b_host)
     assert np.array_equal(s_dev.cpu().numpy().view(np.uint16), np.asarray(s_host).view(np.uint16))
+
+
+@pytest.mark.parametrize("k,n,groupsize", [(256, 256, 128), (2560, 9216, 128), (9216, 2560, 128), (512, 1280, -1)])
+def test_device_gptq_repack_equals_host_repack(oracle, k, n, groupsize):
+    """`kiln_w4a16_repack_gptq_device` against the host repack (pinned on the CPU by the written-layout and
+    round-trip tests): same words, same scales; zero-points other than 8 are refused before anything is written."""
+    q = oracle.np_pack_gptq(oracle.gen_codes(k, n, seed=k + n))
+    s_bits = oracle.gen_scales_f16(k, n, groupsize, seed=k)
+    b_host, s_host = pack.repack_gptq(q, s_bits, None, groupsize)
+    qt = torch.from_numpy(np.asarray(q).view(np.int32)).cuda()
+    st = torch.from_numpy(np.asarray(s_bits).view(np.float16)).cuda()
+    g = k if groupsize == -1 else groupsize
+    zeros = torch.full((k // g, n // 8), -0x77777778, dtype=torch.int32, device="cuda")     # 0x88888888
+    for qz in (None, zeros):
+        b_dev, s_dev = pack.repack_gptq_device(qt, st, qz, groupsize)
+        torch.cuda.synchronize()
+        assert np.array_equal(b_dev.cpu().numpy(), np.asarray(b_host).view(np.int32))
+        assert np.array_equal(s_dev.cpu().numpy().view(np.uint16), np.asarray(s_host).view(np.uint16))
+    bad = zeros.clone()
+    bad[-1, -1] = 0x77777777
+    with pytest.raises(marlin_gemm.MarlinGemmError, match="zero-point"):
+        pack.repack_gptq_device(qt, st, bad, groupsize)
