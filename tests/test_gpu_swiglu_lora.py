@@ -62,6 +62,7 @@ def _problem(oracle, m, k, n_out, gate_ranks, up_ranks, seed, sigma=1.0, sigma_a
     (200, 2560, 2560, (16,), (32,)),        # the matrix-core kernel, 64-row blocks
     (512, 2560, 9216, (16, 32), (16,)),     # ... on the model's MLP
     (1100, 1024, 4096, (16,), (16,)),       # 128-row blocks
+    (2048, 2560, 9216, (16, 16), (16, 16)), # the chunked-prefill configuration's rows on the model's MLP
 ])
 def test_swiglu_lora_cases(oracle, m, k, n_out, gate_ranks, up_ranks):
     sigma = 1.0 if m <= 128 else 0.5
