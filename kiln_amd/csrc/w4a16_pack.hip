@@ -180,6 +180,7 @@ __global__ void w4a16_check_qzeros_kernel(const uint32_t *__restrict__ qzeros, s
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
         if (qzeros[i] != 0x88888888u) *bad = 1;
 }
+__global__ void w4a16_clear_flag_kernel(int *flag) { *flag = 0; }
 
 }  // namespace
 }  // namespace kiln
@@ -200,7 +201,7 @@ extern "C" kiln_marlin_status_t kiln_w4a16_repack_gptq_device(const void *qweigh
         // this one check waits for the stream.  The flag lives at the start of the output and is overwritten below.
         int *flag = reinterpret_cast<int *>(b_packed);
         int bad = 0;
-        if (hipMemsetAsync(flag, 0, sizeof(int), st) != hipSuccess) return KILN_W4A16_ERR_LAUNCH;
+        w4a16_clear_flag_kernel<<<1, 1, 0, st>>>(flag);
         w4a16_check_qzeros_kernel<<<64, 256, 0, st>>>((const uint32_t *)qzeros, (size_t)Gs * (n / 8), flag);
         if (hipGetLastError() != hipSuccess ||
             hipMemcpyAsync(&bad, flag, sizeof(int), hipMemcpyDeviceToHost, st) != hipSuccess ||
