@@ -115,3 +115,40 @@ def test_graph_of_device_pack_and_gemm():
     _replay_and_compare(calls, [o], [x])
     b_ref, s_ref = marlin_gemm.pack.quantize_and_pack_device(w, GROUP)
     assert torch.equal(b, b_ref) and torch.equal(s, s_ref)
+
+
+def test_two_streams_with_their_own_workspaces_do_not_disturb_each_other():
+    """The library has no state besides the caller's workspace: calls on two streams, each with the workspace the
+    wrapper keeps for that stream, may overlap in time -- K-sliced GEMMs and GEMMs with adapters (whose flags and
+    counters live in the workspace prefix) give the bits of the serial run."""
+    m, ranks, scales = 16, (16, 32), (0.5, 1.0)
+    shapes = [(9216, 2560), (2560, 8192)]
+    ws = [_weights(k, n, 20 + i) for i, (k, n) in enumerate(shapes)]
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    ad = [((torch.randn(sum(ranks), k, device="cuda", generator=gen) * 0.05).to(torch.bfloat16),
+           (torch.randn(n, sum(ranks), device="cuda", generator=gen) * 0.05).to(torch.bfloat16)) for k, n in shapes]
+    xs = [[(torch.randn(m, k, device="cuda", generator=gen) * 0.5).to(torch.bfloat16) for k, _ in shapes] for _ in range(2)]
+
+    def run(side, outs):
+        for j, ((b, s), (la, lb)) in enumerate(zip(ws, ad)):
+            marlin_gemm.marlin_w4a16_gemm(xs[side][j], b, s, GROUP, out=outs[2 * j])
+            marlin_gemm.marlin_w4a16_gemm_lora(xs[side][j], b, s, GROUP, la, lb, ranks, scales, out=outs[2 * j + 1])
+
+    def fresh():
+        return [torch.empty(m, n, dtype=torch.bfloat16, device="cuda") for _, n in shapes for _ in range(2)]
+
+    serial = [fresh(), fresh()]
+    for side in range(2):
+        run(side, serial[side])
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for _ in range(20):
+        both = [fresh(), fresh()]
+        for rep in range(4):
+            for side in range(2):
+                with torch.cuda.stream(streams[side]):
+                    run(side, both[side])
+        torch.cuda.synchronize()
+        for side in range(2):
+            for o, e in zip(both[side], serial[side]):
+                assert torch.equal(o.view(torch.int16), e.view(torch.int16))
