@@ -65,7 +65,9 @@ int kiln_marlin_proj_pack_from_bf16_batch(const void *const *weights_t, const in
  * Build a packed projection from GPTQ-canonical host tensors (the one-time
  * offline repack; no re-quantisation).  No counterpart in the reference, which
  * dequantises GPTQ weights to bf16 (crates/kiln-model/src/quantized.rs:70-163)
- * and then re-quantises them (marlin_proj.rs:229).
+ * and then re-quantises them (marlin_proj.rs:229).  The tensors are uploaded as they are
+ * and rearranged on the device (kiln_w4a16_repack_gptq_device); KILN_W4A16_HOST_PACK in
+ * {1, true, yes} rearranges on the host and uploads the result (same bits).
  */
 int kiln_marlin_proj_pack_from_gptq(const int32_t *qweight, const uint16_t *scales_f16, const int32_t *qzeros,
                                     int64_t k, int64_t n, int groupsize, int dev,

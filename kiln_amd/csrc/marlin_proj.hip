@@ -262,6 +262,43 @@ int pack_from_gptq(const int32_t *qweight, const uint16_t *scales_f16, const int
     if (dev < 0 || !shape_is_supported(k, n)) return KILN_PROJ_SKIPPED;
     if (!(groupsize == -1 || groupsize == 128))
         return fail("marlin_proj: groupsize must be -1 or 128 (got " + std::to_string(groupsize) + ")");
+    if (!env_truthy("KILN_W4A16_HOST_PACK")) {
+        // the checkpoint's tensors go to the device as they are and are rearranged there (same bits)
+        if (!qweight || !scales_f16) return fail("marlin_proj: repack: null or inconsistent argument");
+        if (k > INT32_MAX || n > INT32_MAX) return fail("marlin_proj: weight too large");
+        DeviceScope scope(dev);
+        if (!scope.ok) return fail("marlin_proj: upload b_packed to device");
+        const size_t q_bytes = (size_t)k / 8 * n * sizeof(int32_t);
+        const size_t s_bytes = num_groups(k, groupsize) * (size_t)n * sizeof(uint16_t);
+        const size_t z_bytes = qzeros ? num_groups(k, groupsize) * (size_t)(n / 8) * sizeof(int32_t) : 0;
+        void *raw = nullptr;  // qweight | scales | qzeros, each 256-byte aligned
+        const size_t s_off = (q_bytes + 255) / 256 * 256, z_off = s_off + (s_bytes + 255) / 256 * 256;
+        auto w = std::make_unique<kiln_marlin_packed_proj>();
+        w->k = k;
+        w->n = n;
+        w->groupsize = groupsize;
+        w->dev = dev;
+        bool ok = hipMalloc(&raw, z_off + z_bytes + 256) == hipSuccess && hipMalloc(&w->b_packed, q_bytes) == hipSuccess &&
+                  hipMalloc(&w->scales, s_bytes) == hipSuccess;
+        ok = ok && hipMemcpy(raw, qweight, q_bytes, hipMemcpyHostToDevice) == hipSuccess &&
+             hipMemcpy((char *)raw + s_off, scales_f16, s_bytes, hipMemcpyHostToDevice) == hipSuccess &&
+             (!qzeros || hipMemcpy((char *)raw + z_off, qzeros, z_bytes, hipMemcpyHostToDevice) == hipSuccess);
+        int st = KILN_W4A16_ERR_LAUNCH;
+        if (ok) {
+            st = kiln_w4a16_repack_gptq_device(raw, (char *)raw + s_off, qzeros ? (char *)raw + z_off : nullptr, (int)k, (int)n,
+                                               groupsize, w->b_packed, w->scales, dev, nullptr);
+            if (st == KILN_W4A16_OK && hipStreamSynchronize(nullptr) != hipSuccess) st = KILN_W4A16_ERR_LAUNCH;
+        }
+        if (raw) (void)hipFree(raw);
+        if (!ok || st != KILN_W4A16_OK) {
+            if (w->b_packed) (void)hipFree(w->b_packed);
+            if (w->scales) (void)hipFree(w->scales);
+            if (!ok) return fail("marlin_proj: upload b_packed to device");
+            return fail(std::string("marlin_proj: repack: ") + kiln_w4a16_status_string((kiln_marlin_status_t)st));
+        }
+        *out = w.release();
+        return KILN_PROJ_OK;
+    }
     PackedHost p;
     p.k = k;
     p.n = n;

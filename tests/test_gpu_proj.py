@@ -41,10 +41,18 @@ def test_native_batch_pack_keeps_order_and_skips(monkeypatch, oracle):
             assert torch.equal(a.b_packed, b.b_packed) and torch.equal(a.scales, b.scales)
 
 
-def test_native_gptq_repack_and_matmul_ranks(oracle):
+def test_native_gptq_repack_and_matmul_ranks(oracle, monkeypatch):
     m, k, n, g = 24, 2560, 1024, 128
     x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=5)
     b, s = pack.repack_gptq(q, s_bits, None, g)
+    good_zeros = torch.full((k // g, n // 8), -0x77777778, dtype=torch.int32)     # 0x88888888
+    monkeypatch.setenv("KILN_W4A16_HOST_PACK", "1")                                  # the host route of the repack
+    on_host = marlin_proj.pack_from_gptq(torch.from_numpy(q.view(np.int32)), torch.from_numpy(s_bits.view(np.float16)),
+                                         good_zeros, g, "cuda")
+    monkeypatch.delenv("KILN_W4A16_HOST_PACK")
+    proj = marlin_proj.pack_from_gptq(torch.from_numpy(q.view(np.int32)), torch.from_numpy(s_bits.view(np.float16)),
+                                      good_zeros, g, "cuda")
+    assert torch.equal(proj.b_packed, on_host.b_packed) and torch.equal(proj.scales, on_host.scales)
     proj = marlin_proj.pack_from_gptq(torch.from_numpy(q.view(np.int32)), torch.from_numpy(s_bits.view(np.float16)),
                                       None, g, "cuda")
     assert np.array_equal(proj.b_packed.cpu().numpy(), b)
