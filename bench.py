@@ -129,6 +129,39 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
                                             "plain_gemm_same_weights_us": round(t_plain / count * 1e6, 2),
                                             "with_two_lora_adapters_a_side_us": round(t_lora / count * 1e6, 2)}
 
+    # one layer's quantised linears of a decode step at 16 rows -- in-projection, out-projection, fused gate+up
+    # SwiGLU, down -- without adapters and with two stacked adapters on every projection (ranks 16 + 32; 16 + 16 on gate and on up)
+    from kiln_amd.marlin_gemm import interleave_gate_up_lora_b
+    lay = {"in": (2560, 8192), "out": (4096, 2560), "gate_up": (2560, 18432), "down": (9216, 2560)}
+    lw = {name: [make_layer(*kn) for _ in range(8)] for name, kn in lay.items()}
+    lx = {name: torch.randn(16, kn[0], device=dev).to(torch.bfloat16) for name, kn in lay.items()}
+    lo_ = {name: torch.empty(16, kn[1] // (2 if name == "gate_up" else 1), dtype=torch.bfloat16, device=dev)
+           for name, kn in lay.items()}
+    lr, ls = (16, 32), (0.5, 1.0)
+    la_ = {name: (torch.randn(sum(lr), kn[0], device=dev) * 0.02).to(torch.bfloat16) for name, kn in lay.items()}
+    lb_ = {name: (torch.randn(kn[1], sum(lr), device=dev) * 0.02).to(torch.bfloat16) for name, kn in lay.items() if name != "gate_up"}
+    gr, gsc = (16, 16, 16, 16), (0.5, 1.0, 0.5, 1.0)   # gate's two adapters, then up's: 64 rank columns, the fused call's limit
+    gu_a = (torch.randn(sum(gr), 2560, device=dev) * 0.02).to(torch.bfloat16)
+    gu_b = interleave_gate_up_lora_b((torch.randn(9216, 32, device=dev) * 0.02).to(torch.bfloat16),
+                                     (torch.randn(9216, 32, device=dev) * 0.02).to(torch.bfloat16), 9216)
+    def layer_plain(i):
+        for name in ("in", "out"):
+            marlin_gemm.marlin_w4a16_gemm(lx[name], *lw[name][i % 8], GROUP, out=lo_[name])
+        marlin_w4a16_gemm_swiglu(lx["gate_up"], *lw["gate_up"][i % 8], GROUP, out=lo_["gate_up"])
+        marlin_gemm.marlin_w4a16_gemm(lx["down"], *lw["down"][i % 8], GROUP, out=lo_["down"])
+    def layer_lora(i):
+        for name in ("in", "out"):
+            marlin_gemm.marlin_w4a16_gemm_lora(lx[name], *lw[name][i % 8], GROUP, la_[name], lb_[name], lr, ls, out=lo_[name])
+        marlin_w4a16_gemm_swiglu_lora(lx["gate_up"], *lw["gate_up"][i % 8], GROUP, gu_a, gu_b, gr, gsc,
+                                      out=lo_["gate_up"])
+        marlin_gemm.marlin_w4a16_gemm_lora(lx["down"], *lw["down"][i % 8], GROUP, la_["down"], lb_["down"], lr, ls,
+                                           out=lo_["down"])
+    t_p, _ = timed_graph(layer_plain, 64)
+    t_l, _ = timed_graph(layer_lora, 64)
+    extra["decode_layer_m16_four_linears"] = {"us": round(t_p / 64 * 1e6, 2),
+                                              "with_two_lora_adapters_per_projection_us": round(t_l / 64 * 1e6, 2)}
+    del lw
+
     # per-launch distribution and wrapper-inclusive cost of the headline GEMM (eager launches)
     ws_ = [make_layer(2560, 18432) for _ in range(16)]
     x_ = torch.randn(16, 2560, device=dev).to(torch.bfloat16)
