@@ -39,6 +39,10 @@ int kiln_marlin_proj_env_enabled(void);
 /* parallel_pack_disabled (marlin_proj.rs:346-356): KILN_DISABLE_PARALLEL_PACK in {1, true, yes}. */
 int kiln_marlin_proj_parallel_pack_disabled(void);
 
+/* marlin_bf16_drop_disabled (crates/kiln-model/src/forward.rs:1565-1580): KILN_DISABLE_MARLIN_BF16_DROP in
+ * {1, true, yes} keeps the bf16 copy of a projection resident beside its packed weight. */
+int kiln_marlin_proj_bf16_drop_disabled(void);
+
 /*
  * pack_from_bf16 (marlin_proj.rs:198-207): quantise and pack a bf16 [k, n] row-major
  * weight that lies on device `dev`.  The reference downloads it, packs on the host and

@@ -48,6 +48,19 @@ typedef int kiln_marlin_status_t;
 #define KILN_W4A16_ERR_ZERO_POINT   5  /* repack: a GPTQ zero-point other than 8 */
 #define KILN_W4A16_ERR_SCRATCH      6  /* the call needs more scratch than the library's static array holds */
 
+/*
+ * Bits of the workspace's sticky word (kiln_w4a16_workspace_check): which bounded wait gave up.
+ * Launches whose blocks wait for other blocks of the same launch (K slices that meet in the zeroed
+ * prefix, blocks that wait for a LoRA projection computed by the launch's first blocks) poll a bounded
+ * number of times (2^20 polls, tens of milliseconds).  Blocks are dispatched in index order and a
+ * waiting block only waits for lower indices, so a launch that has the GPU to itself always gets there.
+ */
+#define KILN_W4A16_WAIT_DECODE_EXCHANGE 1u   /* K slices of a call of up to 16 rows */
+#define KILN_W4A16_WAIT_MID_EXCHANGE    2u   /* K slices of a call of 33...192 rows */
+#define KILN_W4A16_WAIT_DECODE_FOLD     4u   /* LoRA projection inside a launch of up to 16 rows */
+#define KILN_W4A16_WAIT_MID_FOLD        8u   /* ... of 17...192 rows */
+#define KILN_W4A16_WAIT_PREFILL_FOLD    16u  /* ... on the matrix-core path */
+
 /* Size of the static device array behind kiln_marlin_w4a16_gemm_static_scratch (per GPU). */
 #define KILN_W4A16_STATIC_SCRATCH_BYTES (8u << 20)
 
@@ -97,6 +110,31 @@ size_t kiln_w4a16_workspace_bytes_tuned(int prob_m, int prob_n, int prob_k,
  * marlin_kernel.cu:177-180, lib.rs:176-178).
  */
 size_t kiln_w4a16_workspace_zeroed_bytes(void);
+
+/*
+ * What a caller can learn about the bounded waits, and how it recovers.  No counterpart in the
+ * reference, whose lock waits are unbounded (marlin_kernel.cu:162-175).
+ *
+ * A wavefront whose wait runs out ORs a KILN_W4A16_WAIT_* bit into one word of the workspace
+ * (kiln_w4a16_workspace_error_offset() bytes from its start, inside the zeroed prefix, used by nothing
+ * else) and goes on: the call that gave up returns rows with NaN or without their low-rank term, and
+ * what it was waiting for may land later and leave the prefix non-zero, which would corrupt every later
+ * call on that workspace.  Nothing clears the word but kiln_w4a16_workspace_reset.
+ *   kiln_w4a16_workspace_check  enqueues a 4-byte copy of the word to *host_word on `stream`; after the
+ *       caller has synchronised the stream, 0 means no wait has given up since the last reset.  (A copy
+ *       to host memory: not for use under graph capture.)
+ *   kiln_w4a16_workspace_reset  zero-fills the prefix, sticky word included, with a kernel on `stream`
+ *       (may be captured); call it after a non-zero check, once the stream has drained.
+ * workspace == NULL means the static array of kiln_marlin_w4a16_gemm_static_scratch on the current device.
+ * When can a wait run out?  Only when launches from several streams share the GPU in such a way that
+ * waiting blocks hold every slot of a die while the blocks they wait for are queued behind other
+ * launches' waiting blocks; up to four concurrent streams of the model's shapes cannot get there (a die
+ * never fills with waiting blocks alone), more can in principle.  Serving code that overlaps many GEMM
+ * streams should check the word once per step.
+ */
+size_t kiln_w4a16_workspace_error_offset(void);
+kiln_marlin_status_t kiln_w4a16_workspace_check(const void *workspace, uint32_t *host_word, void *stream);
+kiln_marlin_status_t kiln_w4a16_workspace_reset(void *workspace, void *stream);
 
 /*
  * kiln_marlin_w4a16_gemm without the workspace argument, for callers that cannot allocate

@@ -4,7 +4,12 @@
 // compiles the HIP sources for gfx950 with hipcc and links the HIP runtime.
 // Unlike the reference it fails loudly when the toolkit is missing instead of
 // skipping the kernel.
-use std::{env, path::PathBuf, process::Command};
+//
+// What is compiled is not spelled out here: csrc/objects.list names every object of the library as
+// `object:source[:extra flag]` (some kernel files are compiled twice, the second time with a define
+// that adds the low-rank term), and the Makefile that builds the shared library for the C and
+// Python harnesses reads the same file, so the two builds cannot drift apart.
+use std::{env, fs, path::PathBuf, process::Command};
 
 fn main() {
     let rocm = env::var("ROCM_PATH").unwrap_or_else(|_| "/opt/rocm".into());
@@ -12,32 +17,46 @@ fn main() {
     assert!(hipcc.exists(), "kiln-marlin-gemm: hipcc not found under {rocm}; set ROCM_PATH");
     let arch = env::var("KILN_HIP_ARCHS").unwrap_or_else(|_| "gfx950".into());
     let out = PathBuf::from(env::var("OUT_DIR").unwrap());
-    let csrc = PathBuf::from(env::var("CARGO_MANIFEST_DIR").unwrap()).join("csrc");
+    let crate_dir = PathBuf::from(env::var("CARGO_MANIFEST_DIR").unwrap());
+    // csrc/ holds the kernel sources, include/ the two public headers (kiln_w4a16.h, kiln_marlin_proj.h)
+    let (csrc, include) = (crate_dir.join("csrc"), crate_dir.join("include"));
 
+    let manifest = csrc.join("objects.list");
+    let listing = fs::read_to_string(&manifest).expect("kiln-marlin-gemm: csrc/objects.list is missing");
+    println!("cargo:rerun-if-changed=csrc/objects.list");
     let mut objects = Vec::new();
-    // (source, object, extra define): the small-M kernels are compiled twice, the second time
-    // as the instances that add the low-rank (LoRA) term where they store a tile
-    for (src, obj, define) in [
-        ("w4a16_api.hip", "w4a16_api.o", None),
-        ("w4a16_decode.hip", "w4a16_decode.o", None),
-        ("w4a16_decode.hip", "w4a16_decode_lora.o", Some("-DKILN_DECODE_LORA=1")),
-        ("w4a16_prefill.hip", "w4a16_prefill.o", None),
-        ("marlin_proj.hip", "marlin_proj.o", None),
-        ("pack_host.cpp", "pack_host.o", None),
-    ] {
-        let obj = out.join(obj);
-        let mut cmd = Command::new(&hipcc);
-        cmd.arg(format!("--offload-arch={arch}"))
-            .args(["-O3", "-std=c++17", "-fPIC", "-c"])
-            // packed-f32 VALU instructions are switched off for all device code
-            .args(["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]);
-        if let Some(d) = define {
-            cmd.arg(d);
+    for line in listing.lines().map(str::trim).filter(|l| !l.is_empty() && !l.starts_with('#')) {
+        let mut fields = line.split(':');
+        let (stem, src) = (fields.next().unwrap(), fields.next().expect("object:source[:flag]"));
+        let flag = fields.next();
+        let obj = out.join(format!("{stem}.o"));
+        let mut cmd = if src.ends_with(".cpp") {
+            // host code: the quantiser and the layout writer
+            let mut c = Command::new(env::var("CXX").unwrap_or_else(|_| "g++".into()));
+            c.args(["-O3", "-std=c++17", "-fPIC", "-pthread", "-c"]);
+            c
+        } else {
+            let mut c = Command::new(&hipcc);
+            c.arg(format!("--offload-arch={arch}"))
+                .args(["-O3", "-std=c++17", "-fPIC", "-c"])
+                // packed-f32 VALU instructions are switched off for all device code
+                .args(["-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]);
+            c
+        };
+        cmd.arg(format!("-I{}", include.display()));
+        if let Some(f) = flag {
+            cmd.arg(f);
         }
         cmd.arg(csrc.join(src)).arg("-o").arg(&obj);
-        assert!(cmd.status().expect("run hipcc").success(), "hipcc failed on {src}");
+        assert!(cmd.status().expect("run the compiler").success(), "compiling {src} failed");
         println!("cargo:rerun-if-changed=csrc/{src}");
         objects.push(obj);
+    }
+    assert!(!objects.is_empty(), "kiln-marlin-gemm: csrc/objects.list names no object");
+    for entry in fs::read_dir(&csrc).unwrap().flatten() {
+        if entry.path().extension().is_some_and(|e| e == "h") {
+            println!("cargo:rerun-if-changed=csrc/{}", entry.file_name().to_string_lossy());
+        }
     }
     let lib = out.join("libkiln_marlin_gemm.a");
     assert!(Command::new("ar").arg("crs").arg(&lib).args(&objects).status().unwrap().success());

@@ -33,6 +33,10 @@ unsafe extern "C" {
         weight: *const f32, k: i32, n: i32, groupsize: i32,
         b_packed: *mut i32, scales_f16: *mut u16, dequant: *mut f32,
     ) -> i32;
+    fn kiln_w4a16_quantize_and_pack_device(
+        weight_bf16: *const c_void, k: i32, n: i32, groupsize: i32,
+        b_packed: *mut c_void, scales_f16: *mut c_void, dev: i32, stream: *mut c_void,
+    ) -> i32;
 }
 
 macro_rules! device_slice {
@@ -113,6 +117,36 @@ fn workspace_for(a: &Tensor, m: usize, n: usize, k: usize) -> Result<Tensor> {
     } else { head };
     cache.insert(key, ws.clone());
     Ok(ws)
+}
+
+/// Quantise and pack a bf16 `[k, n]` weight where it lies, on the GPU: the bits `pack::quantize_and_pack`
+/// gives for the same values, without the download, host pack and upload.  A caller that holds the weight
+/// on the device (`kiln-model/src/marlin_proj.rs:86-181` does) calls this instead of the three phases.
+/// Returns `(b_packed [k/16, 2n] i32, scales [k/g, n] f16)`.
+pub fn quantize_and_pack_device(weight_bf16: &Tensor, groupsize: i32) -> Result<(Tensor, Tensor)> {
+    let (k, n) = weight_bf16.dims2()?;
+    if k % 128 != 0 || n % 256 != 0 { candle_core::bail!("kiln-marlin-gemm: weight [{k}, {n}] needs k % 128 == 0 and n % 256 == 0"); }
+    if groupsize != -1 && groupsize != 128 { candle_core::bail!("kiln-marlin-gemm: groupsize must be -1 or 128 (got {groupsize})"); }
+    if weight_bf16.dtype() != DType::BF16 { candle_core::bail!("kiln-marlin-gemm: weight must be bf16 (got {:?})", weight_bf16.dtype()); }
+    let w = weight_bf16.contiguous()?;
+    let groups = if groupsize == -1 { 1 } else { k / 128 };
+    let b_packed = unsafe { Tensor::empty((k / 16, n * 2), DType::I32, w.device())? };
+    let scales = unsafe { Tensor::empty((groups, n), DType::F16, w.device())? };
+    {
+        let (w_s, dev) = device_slice!(w, bf16, "weight");
+        let (b_s, _) = device_slice!(b_packed, i32, "b_packed");
+        let (s_s, _) = device_slice!(scales, f16, "scales");
+        let stream = dev.cuda_stream();
+        let status = unsafe {
+            let (wp, _g0) = w_s.device_ptr(&stream);
+            let (bp, _g1) = b_s.device_ptr(&stream);
+            let (sp, _g2) = s_s.device_ptr(&stream);
+            kiln_w4a16_quantize_and_pack_device(wp as *const _, k as i32, n as i32, groupsize, bp as *mut _, sp as *mut _,
+                dev.ordinal() as i32, stream.cu_stream() as *mut c_void)
+        };
+        if status != 0 { candle_core::bail!("kiln_w4a16_quantize_and_pack_device failed with status {status} for k={k}, n={n}"); }
+    }
+    Ok((b_packed, scales))
 }
 
 pub mod pack {

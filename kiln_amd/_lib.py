@@ -16,6 +16,9 @@ EXPORTS = (
     "kiln_w4a16_workspace_bytes",
     "kiln_w4a16_workspace_bytes_tuned",
     "kiln_w4a16_workspace_zeroed_bytes",
+    "kiln_w4a16_workspace_error_offset",
+    "kiln_w4a16_workspace_check",
+    "kiln_w4a16_workspace_reset",
     "kiln_marlin_w4a16_gemm_static_scratch",
     "kiln_w4a16_gemm_lora",
     "kiln_w4a16_gemm_swiglu",
@@ -38,6 +41,7 @@ PROJ_EXPORTS = (
     "kiln_marlin_proj_shape_is_supported",
     "kiln_marlin_proj_env_enabled",
     "kiln_marlin_proj_parallel_pack_disabled",
+    "kiln_marlin_proj_bf16_drop_disabled",
     "kiln_marlin_proj_pack_from_bf16",
     "kiln_marlin_proj_pack_from_bf16_batch",
     "kiln_marlin_proj_pack_from_gptq",
@@ -61,6 +65,8 @@ PROJ_OK, PROJ_SKIPPED, PROJ_ERR = 0, 1, -1
 STATIC_SCRATCH_BYTES = 8 << 20   # KILN_W4A16_STATIC_SCRATCH_BYTES
 
 OK, ERR_PROB_SHAPE, ERR_KERN_SHAPE, ERR_LAUNCH, ERR_ARGUMENT, ERR_ZERO_POINT, ERR_SCRATCH = range(7)
+# bits of the workspace's sticky word (KILN_W4A16_WAIT_*): which bounded wait gave up
+WAIT_DECODE_EXCHANGE, WAIT_MID_EXCHANGE, WAIT_DECODE_FOLD, WAIT_MID_FOLD, WAIT_PREFILL_FOLD = 1, 2, 4, 8, 16
 
 # The tuning build: the same sources with -DKILN_W4A16_TUNING_HOOKS, which adds process-wide
 # overrides of the automatic plan (kiln_w4a16_debug_*).  Tests and profiling scripts that pin a
@@ -141,6 +147,12 @@ def _load(tuning: bool) -> ctypes.CDLL:
     L.kiln_w4a16_workspace_bytes_tuned.argtypes = [i, i, i, i, i, i]
     L.kiln_w4a16_workspace_zeroed_bytes.restype = c.c_size_t
     L.kiln_w4a16_workspace_zeroed_bytes.argtypes = []
+    L.kiln_w4a16_workspace_error_offset.restype = c.c_size_t
+    L.kiln_w4a16_workspace_error_offset.argtypes = []
+    L.kiln_w4a16_workspace_check.restype = i
+    L.kiln_w4a16_workspace_check.argtypes = [vp, c.POINTER(c.c_uint32), vp]
+    L.kiln_w4a16_workspace_reset.restype = i
+    L.kiln_w4a16_workspace_reset.argtypes = [vp, vp]
     L.kiln_marlin_w4a16_gemm_static_scratch.restype = i
     L.kiln_marlin_w4a16_gemm_static_scratch.argtypes = [vp, vp, vp, vp, i, i, i, i, i, vp]
     L.kiln_w4a16_debug_decode_plan.restype = i
@@ -184,6 +196,8 @@ def _load(tuning: bool) -> ctypes.CDLL:
     L.kiln_marlin_proj_env_enabled.argtypes = []
     L.kiln_marlin_proj_parallel_pack_disabled.restype = i
     L.kiln_marlin_proj_parallel_pack_disabled.argtypes = []
+    L.kiln_marlin_proj_bf16_drop_disabled.restype = i
+    L.kiln_marlin_proj_bf16_drop_disabled.argtypes = []
     L.kiln_marlin_proj_pack_from_bf16.restype = i
     L.kiln_marlin_proj_pack_from_bf16.argtypes = [vp, i64, i64, i, i, pp]
     L.kiln_marlin_proj_pack_from_bf16_batch.restype = i

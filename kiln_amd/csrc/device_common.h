@@ -3,6 +3,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include "launch.h"
 #include "layout.h"
 
 namespace kiln {
@@ -105,6 +106,19 @@ __device__ __forceinline__ void store_tile_rows(uint16_t *__restrict__ C, int N,
                 dst[(size_t)i * n_out] = f32_to_bf16_bits(gate * __builtin_amdgcn_rcpf(1.f + __expf(-gate)) * up[i]);
             }
     }
+}
+
+// A bounded wait ran out: leave a mark the host can find (launch.h describes the word).  `exchange_region`
+// is the start of the region in which K slices meet without counters, `fold_words` the LoRA fold's flags;
+// both sit at fixed distances from the sticky word.  One lane; the wavefront goes on with what it has.
+__device__ __forceinline__ void report_wait_gave_up(unsigned *error_word, unsigned which, int lane) {
+    if (lane == 0) __hip_atomic_fetch_or(error_word, which, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned *error_word_before_exchange_region(const void *exchange_region) {
+    return reinterpret_cast<unsigned *>(reinterpret_cast<uintptr_t>(exchange_region) - (kWsCounterBytes - kWsErrorOffset));
+}
+__device__ __forceinline__ unsigned *error_word_before_fold_words(const unsigned *fold_words) {
+    return reinterpret_cast<unsigned *>(reinterpret_cast<uintptr_t>(fold_words) - (kWsFoldFlagOffset - kWsErrorOffset));
 }
 
 __device__ __forceinline__ bf16x8 bf16x8_zero() {

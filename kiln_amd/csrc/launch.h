@@ -7,6 +7,28 @@
 
 namespace kiln {
 
+// The start of every workspace, zero whenever no launch is running:
+//   [0, 64 KiB)          arrival counters of the exchanges that count; the last 64 bytes are not a
+//                        counter but one sticky word (kWsErrorOffset): a wavefront whose bounded wait ran
+//                        out ORs a bit into it (which wait: the enum below) and nothing ever clears it but
+//                        the caller, so that a launch that gave up can be told from one that worked
+//   [64 KiB, + 4 MiB)    the region in which K slices exchange partial tiles that are their own arrival
+//                        flags; its last 64 KiB hold the flags and counts of a LoRA projection folded
+//                        into its GEMM's launch (16 replicas, 4 KiB apart: lora_tail.h)
+constexpr size_t kWsCounterBytes = 64 * 1024;
+constexpr size_t kWsErrorOffset = kWsCounterBytes - 64;
+constexpr size_t kWsCounterCapacity = kWsErrorOffset;  // bytes of the counter region that hold counters
+constexpr size_t kWsFlaggedBytes = 4 * 1024 * 1024;
+constexpr size_t kWsFoldFlagBytes = 16 * 4096;
+constexpr size_t kWsFoldFlagOffset = kWsCounterBytes + kWsFlaggedBytes - kWsFoldFlagBytes;
+enum WaitGaveUp : unsigned {
+    kGaveUpDecodeExchange = 1u,  // K slices of a launch of up to 16 rows
+    kGaveUpMidExchange = 2u,     // K slices of a launch of 33...192 rows
+    kGaveUpDecodeFold = 4u,      // a block of up to 16 rows waiting for the folded LoRA projection
+    kGaveUpMidFold = 8u,         // the same at 17...192 rows
+    kGaveUpPrefillFold = 16u,    // the same on the matrix-core path
+};
+
 // One launch of the decode kernel: M <= 16 rows of A against the whole weight.
 constexpr int kDecodeFlaggedMaxSlices = 4;
 

@@ -35,7 +35,13 @@
 
 namespace kiln {
 
-constexpr int kLayoutVersion = 1;
+// Revision of the layout written into artefacts.
+//   1: the chunk layout of this file; fused gate/up packs carried 32 gate then 32 up columns per 64.
+//   2: fused gate/up packs carry 8 gate then the 8 matching up columns per 16-column tile, which is
+//      what every kernel's SwiGLU store pairs up.  The chunk layout itself did not change, but a
+//      revision-1 fused pack read by these kernels would pair the wrong columns without any error,
+//      so revision-1 artefacts are refused and must be repacked.
+constexpr int kLayoutVersion = 2;
 constexpr int kTileN = 16;        // columns per chunk
 constexpr int kGroupK = 128;      // rows per chunk (= quantisation group)
 constexpr int kChunkWords = 256;  // 1 KiB

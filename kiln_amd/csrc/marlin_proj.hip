@@ -17,8 +17,8 @@
 #include <thread>
 #include <vector>
 
-#include "../../include/kiln_marlin_proj.h"
-#include "../../include/kiln_w4a16.h"
+#include "kiln_marlin_proj.h"
+#include "kiln_w4a16.h"
 
 struct kiln_marlin_packed_proj {
     void *b_packed = nullptr;  // device, int32 [k/16, 2n]
@@ -476,6 +476,7 @@ using namespace kiln::proj;
 int kiln_marlin_proj_shape_is_supported(int64_t k, int64_t n) { return shape_is_supported(k, n) ? 1 : 0; }
 int kiln_marlin_proj_env_enabled(void) { return env_truthy("KILN_W4A16") ? 1 : 0; }
 int kiln_marlin_proj_parallel_pack_disabled(void) { return env_truthy("KILN_DISABLE_PARALLEL_PACK") ? 1 : 0; }
+int kiln_marlin_proj_bf16_drop_disabled(void) { return env_truthy("KILN_DISABLE_MARLIN_BF16_DROP") ? 1 : 0; }
 
 int kiln_marlin_proj_pack_from_bf16(const void *weight_t, int64_t k, int64_t n, int groupsize, int dev,
                                     kiln_marlin_packed_proj_t **out) {

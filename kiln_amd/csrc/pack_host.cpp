@@ -11,7 +11,7 @@
 #include <thread>
 #include <vector>
 
-#include "../../include/kiln_w4a16.h"
+#include "kiln_w4a16.h"
 #include "layout.h"
 
 namespace {
@@ -162,7 +162,11 @@ kiln_marlin_status_t kiln_w4a16_quantize_and_pack(const float *weight, int k, in
                                 else if (q >= 2147483647.0f) raw = 2147483647LL;
                                 else if (q <= -2147483648.0f) raw = -2147483648LL;
                                 else raw = (long long)q;
-                                const int code = (int)std::min<long long>(15, std::max<long long>(0, raw + 8));
+                                // the reference adds the offset in i32 (lib.rs:423): from a saturated raw a
+                                // release build wraps to a negative sum, which the clamp makes code 0
+                                long long shifted = raw + 8;
+                                if (shifted > 2147483647LL) shifted -= 4294967296LL;
+                                const int code = (int)std::min<long long>(15, std::max<long long>(0, shifted));
                                 words[c] |= (uint32_t)code << (4 * nibble_pos(j));
                                 if (drow) drow[c] = (float)(code - 8) * s_f32[c];
                             }

@@ -4,7 +4,7 @@
 #include <mutex>
 #include <unordered_map>
 
-#include "../../include/kiln_w4a16.h"
+#include "kiln_w4a16.h"
 #include "device_common.h"
 #include "launch.h"
 
@@ -13,16 +13,15 @@ namespace kiln {
 namespace {
 
 constexpr int kMaxDevices = 16;
-constexpr size_t kCounterBytes = 64 * 1024;   // arrival counters at the start of the workspace
-// Behind the counters: the region in which K slices exchange partial tiles without counters.  It is
-// all zero whenever no launch is running (the caller zero-fills it once with the counters; the
-// wavefront that adds a tile's parts writes zeros back), and a written word is never zero.
-constexpr size_t kFlaggedBytes = 4 * 1024 * 1024;
+// The workspace prefix that is zero between launches (launch.h): counters and the sticky word of the
+// bounded waits, then the region in which K slices exchange partial tiles without counters, whose end
+// holds the flags and counts of a LoRA projection folded into its GEMM's launch.
+constexpr size_t kCounterBytes = kWsCounterBytes;
+constexpr size_t kCounterCapacity = kWsCounterCapacity;  // what counters may use of it
+constexpr size_t kFlaggedBytes = kWsFlaggedBytes;
 constexpr size_t kZeroedBytes = kCounterBytes + kFlaggedBytes;
-// the end of that region: producer flags and reader counts of a LoRA projection folded into its GEMM
-// launch (16 replicas, 4 KiB apart: lora_tail.h)
-constexpr size_t kFoldFlagBytes = 16 * 4096;
-constexpr size_t kFoldFlagOffset = kCounterBytes + kFlaggedBytes - kFoldFlagBytes;
+constexpr size_t kFoldFlagBytes = kWsFoldFlagBytes;
+constexpr size_t kFoldFlagOffset = kWsFoldFlagOffset;
 
 struct DeviceInfo {
     std::once_flag once;
@@ -92,7 +91,7 @@ PrefillPlan planned_prefill(int m, int n, int k, int cus) {
         p.ks = (G + gsb - 1) / gsb;
     }
     // one arrival counter per sliced tile lives in the counter region
-    if ((size_t)((m + p.bm - 1) / p.bm) * (n / p.bn - p.nb_full) * sizeof(int) > kCounterBytes) p.ks = 1;
+    if ((size_t)((m + p.bm - 1) / p.bm) * (n / p.bn - p.nb_full) * sizeof(int) > kCounterCapacity) p.ks = 1;
     return p;
 }
 
@@ -503,7 +502,7 @@ MidPlan plan_mid(int m, int n, int k, int cus) {
             a.pairs = pairs;
             if (!mid_plan_ok(a)) continue;
             const int col_blocks = mid_column_blocks(a);
-            if ((size_t)runs * col_blocks * sizeof(int) > kCounterBytes) continue;
+            if ((size_t)runs * col_blocks * sizeof(int) > kCounterCapacity) continue;
             const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
             const float exchange = ks == 1 ? 0.f : (mid_flagged(a) ? 1.7f * ks - 2.9f : 1.7f * ks - 1.9f);
             const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange;
@@ -550,7 +549,7 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
         }
     }
     // the small-M kernels keep one arrival counter per column tile (and run) in the counter region
-    const bool counters_fit = (size_t)(n / kTileN) * sizeof(int) <= kCounterBytes;
+    const bool counters_fit = (size_t)(n / kTileN) * sizeof(int) <= kCounterCapacity;
     if (!counters_fit || takes_prefill(m, n, k, cus)) return plan_as_prefill(m, n, k, cus, thread_k, thread_n, gp);
     // Runs of A, one launch each -- launches on one stream run in order, so they may share the
     // workspace -- of 16 rows, or of up to 32 where the plan fits the kernel instance that takes two
@@ -577,7 +576,7 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
         l.direct = c.direct;
         l.rows = 0;
         int max_runs = kMaxKSlices / l.plan.KS < 4 ? kMaxKSlices / l.plan.KS : 4;
-        if ((size_t)max_runs * (n / kTileN) * sizeof(int) > kCounterBytes) max_runs = 1;
+        if ((size_t)max_runs * (n / kTileN) * sizeof(int) > kCounterCapacity) max_runs = 1;
         if (g_tune.decode_runs_per_launch > 0 && max_runs > g_tune.decode_runs_per_launch)
             max_runs = g_tune.decode_runs_per_launch;
         int step = l.M;
@@ -643,6 +642,12 @@ __global__ void dequant_f32_kernel(const u32x4 *__restrict__ B, const uint16_t *
             const int kk = g * kGroupK + 32 * t + 8 * kq + j;
             out[(size_t)kk * N + nt * kTileN + c] = (float)(code - 8) * s;   // lib.rs:425
         }
+}
+
+// zero-fill in 16-byte units (a kernel, not a memset: callers may record it into a graph)
+__global__ void zero_fill_kernel(u32x4 *__restrict__ dst, size_t units) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < units; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = u32x4{0u, 0u, 0u, 0u};
 }
 
 }  // namespace
@@ -972,6 +977,33 @@ kiln_marlin_status_t kiln_marlin_w4a16_gemm(const void *A, const void *B, void *
     (void)max_par;
     return gemm_any(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream, thread_k, thread_n, sms,
                     nullptr);
+}
+
+// ---- the sticky word of the bounded waits ---------------------------------------------------------
+// workspace == nullptr: the current device's static array (kiln_marlin_w4a16_gemm_static_scratch).
+static char *workspace_or_static(const void *workspace) {
+    if (workspace) return reinterpret_cast<char *>(const_cast<void *>(workspace));
+    int current = -1;
+    if (hipGetDevice(&current) != hipSuccess || current < 0 || current >= kMaxDevices) return nullptr;
+    return reinterpret_cast<char *>(static_scratch_ptr(current));
+}
+
+size_t kiln_w4a16_workspace_error_offset(void) { return kWsErrorOffset; }
+
+kiln_marlin_status_t kiln_w4a16_workspace_check(const void *workspace, uint32_t *host_word, void *stream) {
+    if (!host_word) return KILN_W4A16_ERR_ARGUMENT;
+    const char *ws = workspace_or_static(workspace);
+    if (!ws) return KILN_W4A16_ERR_ARGUMENT;
+    return hipMemcpyAsync(host_word, ws + kWsErrorOffset, sizeof(uint32_t), hipMemcpyDeviceToHost,
+                          reinterpret_cast<hipStream_t>(stream)) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+}
+
+kiln_marlin_status_t kiln_w4a16_workspace_reset(void *workspace, void *stream) {
+    char *ws = workspace_or_static(workspace);
+    if (!ws) return KILN_W4A16_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(ws) % 16 != 0) return KILN_W4A16_ERR_ARGUMENT;
+    zero_fill_kernel<<<256, 256, 0, reinterpret_cast<hipStream_t>(stream)>>>(reinterpret_cast<u32x4 *>(ws), kZeroedBytes / 16);
+    return hipGetLastError() == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
 }
 
 // The small-M plan for a run of m rows on a part with `cus` compute units (a pure query, no GPU

@@ -421,7 +421,9 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
                         live_tiles * kTileN * lo.r_total / 8, lane);
             if (fold.producers > 0) {
                 KILN_GMP_TL(3, KILN_GMP_NOW());
-                [[maybe_unused]] const int polls = lora_fold_wait(fold, tf / T, lane);
+                const int polls = lora_fold_wait(fold, tf / T, lane);
+                if (__builtin_expect(polls == kLoraFoldSpinLimit, 0))
+                    report_wait_gave_up(error_word_before_fold_words(fold.flags), kGaveUpDecodeFold, lane);
                 KILN_GMP_TL(4, KILN_GMP_NOW());
                 KILN_GMP_TL(5, (long long)polls + 1);
                 lds_signal_store(lora_ready_addr(), kGmpLooked);
@@ -497,8 +499,12 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
                 }
                 // the bound is never reached in a working launch; past it the words still missing read
                 // as NaN in the result
-                if (__builtin_amdgcn_ballot_w64(missing) == 0 || spins == kGmpSpinLimit) {
+                if (__builtin_amdgcn_ballot_w64(missing) == 0) {
                     KILN_GMP_TL(5, (long long)spins + 1);
+                    break;
+                }
+                if (__builtin_expect(spins == kGmpSpinLimit, 0)) {  // the host can see this in the workspace's sticky word
+                    report_wait_gave_up(error_word_before_exchange_region(partial), kGaveUpDecodeExchange, lane);
                     break;
                 }
                 __builtin_amdgcn_s_sleep(2);

@@ -397,13 +397,16 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             if (wave == 0) {
                 const int t0 = zr >> 4, nt = min((M + 15) >> 4, lo.row_tiles - t0), consumer = bz * ncb + bx;
                 const unsigned *mine = lo.words + (consumer % kLoraFoldReplicas) * kLoraFoldReplicaWords + kMidFoldTileWord;
-                for (int spins = 0; spins < kMidFoldSpinLimit; ++spins) {
+                int spins = 0;
+                for (; spins < kMidFoldSpinLimit; ++spins) {
                     unsigned f = 1u;
                     if ((lane >> 2) < lo.slices && (lane & 3) < nt)
                         f = __hip_atomic_load(mine + (lane >> 2) * lo.row_tiles + t0 + (lane & 3), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     if (__builtin_amdgcn_ballot_w64(f == 0u) == 0) break;
                     __builtin_amdgcn_s_sleep(4);
                 }
+                if (__builtin_expect(spins == kMidFoldSpinLimit, 0))
+                    report_wait_gave_up(error_word_before_fold_words(lo.words), kGaveUpMidFold, lane);
                 // count: the replica's count, then the top count; the last block zeroes words and counts
                 const int replica = consumer % kLoraFoldReplicas;
                 const unsigned quota = (unsigned)(lo.consumers - replica + kLoraFoldReplicas - 1) / kLoraFoldReplicas;
@@ -575,7 +578,11 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                     missing |= s2 < KS - 1 && (g.x == 0 || g.y == 0 || g.z == 0 || g.w == 0);
                 }
             // the bound is never reached in a working launch; past it the missing words read as NaN
-            if (__builtin_amdgcn_ballot_w64(missing) == 0 || spins == kMidSpinLimit) break;
+            if (__builtin_amdgcn_ballot_w64(missing) == 0) break;
+            if (__builtin_expect(spins == kMidSpinLimit, 0)) {  // the host can see this in the workspace's sticky word
+                report_wait_gave_up(error_word_before_exchange_region(partial), kGaveUpMidExchange, lane);
+                break;
+            }
             __builtin_amdgcn_s_sleep(2);
         }
 #pragma unroll

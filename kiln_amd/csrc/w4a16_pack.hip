@@ -12,7 +12,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
-#include "../../include/kiln_w4a16.h"
+#include "kiln_w4a16.h"
 #include "device_common.h"
 #include "layout.h"
 
@@ -118,7 +118,8 @@ __global__ __launch_bounds__(256) void w4a16_pack_codes_kernel(const uint16_t *_
             else if (q >= 2147483647.0f) raw = 2147483647LL;
             else if (q <= -2147483648.0f) raw = -2147483648LL;
             else raw = (long long)q;
-            long long code = raw + 8;
+            long long code = raw + 8;  // an i32 sum in the reference (lib.rs:423): wraps from a saturated raw
+            if (code > 2147483647LL) code -= 4294967296LL;
             code = code < 0 ? 0 : (code > 15 ? 15 : code);
             word |= (uint32_t)code << (4 * nibble_pos(j));
         }

@@ -163,12 +163,15 @@ constexpr int kPrefillFoldSpinLimit = 1 << 20;
 // rows [m0, m0 + rows) of T and of the extension operand are in memory
 __device__ __forceinline__ void prefill_fold_wait(const PrefillFold &pf, int m0, int rows, int lane) {
     const int t0 = m0 >> 4, nt = min((rows + 15) >> 4, pf.row_tiles - t0);
-    for (int spins = 0; spins < kPrefillFoldSpinLimit; ++spins) {
+    int spins = 0;
+    for (; spins < kPrefillFoldSpinLimit; ++spins) {
         unsigned f = 1u;
         if (lane < nt) f = __hip_atomic_load(pf.words + kPrefillFoldTileWord + t0 + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (__builtin_amdgcn_ballot_w64(f == 0u) == 0) break;
         __builtin_amdgcn_s_sleep(8);
     }
+    if (__builtin_expect(spins == kPrefillFoldSpinLimit, 0))
+        report_wait_gave_up(error_word_before_fold_words(pf.words), kGaveUpPrefillFold, lane);
 }
 // one wavefront of block `consumer`, after its look: count the block; the last one zeroes everything
 __device__ __forceinline__ void prefill_fold_done(const PrefillFold &pf, int consumer, int lane) {
@@ -749,7 +752,7 @@ size_t prefill_aext_bytes(int m, int k) { return (size_t)m * (k / kGroupK) * siz
 // For the matrix-core kernel: T once and behind it the f32 tiles in which the slices meet (at most
 // ceil(256 / row tiles) slices per row tile: fewer than 256 + 2 x row tiles tiles of 64 or 16 rows
 // x 64 columns).
-constexpr int kProjectMaxCounters = 16384;
+constexpr int kProjectMaxCounters = (int)(kWsCounterCapacity / sizeof(int));  // the counter region less its sticky word
 constexpr int kProjectFoldCounters = 8192;  // folded into the product's launch: the product's counters first, then the projection's
 // measured at 2048 rows: 16-row blocks 9.9 us against 13.1 for K = 2560, 23.5 against 20.2 for K = 9216
 int lora_project_rows_per_block(int m, int k) { return m > 1024 && k > 4096 ? 64 : 16; }
@@ -1019,7 +1022,7 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         project_slicing(a.M, a.K, a.counters != nullptr, &rb, &row_tiles, &kz, &per_slice);
         const int sliced_tiles = (a.N / a.bn - a.nb_full) * ((a.M + a.bm - 1) / a.bm);
         fold = a.lora_words && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
-               a.counters && row_tiles <= kPrefillFoldMaxTiles && row_tiles <= kProjectFoldCounters &&
+               a.counters && row_tiles <= kPrefillFoldMaxTiles && row_tiles <= kProjectMaxCounters - kProjectFoldCounters &&
                sliced_tiles <= kProjectFoldCounters && a.n_adapters >= 1 && a.n_adapters <= 8 && a.lora_a && a.lora_t &&
                a.ranks && a.scales && a.r_total <= kProjectMaxRank;
         if (fold) {

@@ -113,16 +113,20 @@ def queue_layer(layer_idx: int, layer: LayerProjections, kinds: Optional[Sequenc
     return inputs, meta
 
 
-def install_packed(layer: LayerProjections, kind: PackKind, packed: MarlinPackedProj, drop_bf16: bool = True) -> None:
+def install_packed(layer: LayerProjections, kind: PackKind, packed: MarlinPackedProj,
+                   drop_bf16: Optional[bool] = None) -> None:
     """`install_marlin_packed` (forward.rs:1736-1771): the packed weight goes into its slot and the
-    bf16 copy is dropped unless `drop_bf16` is off (`KILN_DISABLE_MARLIN_BF16_DROP`)."""
+    bf16 copy is dropped -- unless the caller says otherwise or, with `drop_bf16` left at None, the
+    environment does (`KILN_DISABLE_MARLIN_BF16_DROP`, forward.rs:1565-1580)."""
+    if drop_bf16 is None:
+        drop_bf16 = not marlin_proj.bf16_drop_disabled()
     layer.packed[kind] = packed
     if drop_bf16:
         layer.weights_t[kind] = None
 
 
 def pack_layers(layers: Sequence[LayerProjections], kinds: Optional[Sequence[PackKind]] = None,
-                groupsize: int = 128, drop_bf16: bool = True, fuse_gate_up: bool = False) -> Dict[str, int]:
+                groupsize: int = 128, drop_bf16: Optional[bool] = None, fuse_gate_up: bool = False) -> Dict[str, int]:
     """The post-loop batch pack and install (forward.rs:2040-2085): every queued projection goes
     through `pack_from_bf16_batch` (serial copies, threaded host pack); a projection whose shape the
     kernels do not take (`shape_is_supported`, e.g. the 32-column `in_proj_a` / `in_proj_b`) comes

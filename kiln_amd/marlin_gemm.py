@@ -42,6 +42,40 @@ def _workspace(device: torch.device, stream_ptr: int, nbytes: int) -> torch.Tens
     return ws
 
 
+def workspace_wait_status(device: torch.device | None = None) -> int:
+    """OR of the sticky words of every workspace this module holds on `device` (all devices if None):
+    0 unless a bounded wait inside some launch gave up (`_lib.WAIT_*` says which kind).  Synchronises
+    the streams involved; meant for a health check once per step or per request, not per GEMM."""
+    import ctypes
+    lib, bits = _lib.load(), 0
+    for (dev_index, stream_ptr), ws in list(_workspaces.items()):
+        if device is not None and device.index is not None and device.index != dev_index:
+            continue
+        word = ctypes.c_uint32(0)
+        with torch.cuda.device(dev_index):
+            st = lib.kiln_w4a16_workspace_check(ws.data_ptr(), ctypes.byref(word), stream_ptr)
+            if st != 0:
+                raise MarlinGemmError(f"kiln_w4a16_workspace_check: {_lib.status_string(st)}")
+            torch.cuda.synchronize(dev_index)
+        bits |= word.value
+    return bits
+
+
+def workspace_reset(device: torch.device | None = None) -> None:
+    """Zero the prefix (sticky word included) of every workspace this module holds on `device`: what a
+    caller does after `workspace_wait_status` came back non-zero and the device has drained."""
+    lib = _lib.load()
+    for (dev_index, stream_ptr), ws in list(_workspaces.items()):
+        if device is not None and device.index is not None and device.index != dev_index:
+            continue
+        with torch.cuda.device(dev_index):
+            torch.cuda.synchronize(dev_index)
+            st = lib.kiln_w4a16_workspace_reset(ws.data_ptr(), stream_ptr)
+            if st != 0:
+                raise MarlinGemmError(f"kiln_w4a16_workspace_reset: {_lib.status_string(st)}")
+            torch.cuda.synchronize(dev_index)
+
+
 def _check_gemm_args(a, b_packed, scales, groupsize):
     """lib.rs:103-166, same order, same texts."""
     if not a.is_cuda:

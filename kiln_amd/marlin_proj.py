@@ -271,3 +271,8 @@ def env_enabled() -> bool:
 def parallel_pack_disabled() -> bool:
     """`KILN_DISABLE_PARALLEL_PACK` (marlin_proj.rs:346-356)."""
     return bool(_lib.load().kiln_marlin_proj_parallel_pack_disabled())
+
+
+def bf16_drop_disabled() -> bool:
+    """`KILN_DISABLE_MARLIN_BF16_DROP` in {1, true, yes} (forward.rs:1565-1580)."""
+    return bool(_lib.load().kiln_marlin_proj_bf16_drop_disabled())

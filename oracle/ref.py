@@ -271,8 +271,13 @@ def np_quantize(w: np.ndarray, groupsize: int):
     s_full = np.repeat(s, g, axis=0)
     with np.errstate(divide="ignore", invalid="ignore"):
         q = np_round_half_away((w / s_full).astype(np.float32))
-    q = np.nan_to_num(q, nan=0.0, posinf=2147483647.0, neginf=-2147483648.0)
-    codes = np.clip(q.astype(np.int64) + 8, 0, 15).astype(np.int32)
+    # `as i32` saturates, NaN -> 0; the i32 sum `raw + Q_OFFSET` (lib.rs:423) wraps in a release build
+    # where raw saturated at i32::MAX (w / s = +inf), and the clamp then gives code 0
+    raw = np.clip(np.nan_to_num(q.astype(np.float64), nan=0.0, posinf=2147483647.0, neginf=-2147483648.0),
+                  -2147483648.0, 2147483647.0).astype(np.int64)
+    shifted = raw + 8
+    shifted = np.where(shifted > 2147483647, shifted - 4294967296, shifted)
+    codes = np.clip(shifted, 0, 15).astype(np.int32)
     deq = ((codes - 8).astype(np.float32) * s_full).astype(np.float32)
     return codes, s_bits, deq
 

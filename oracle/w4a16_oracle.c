@@ -134,8 +134,12 @@ void ko_quantize(const float *weight, int k, int n, int groupsize, int32_t *code
         for (int col = 0; col < n; ++col) {
             const float s = scales[(size_t)grp * n + col];
             /* Rust f32::round = half away from zero = roundf; `as i32`
-             * saturates and maps NaN to 0.  The sum is done in 64 bits so a
-             * saturated value cannot wrap before the clamp. */
+             * saturates and maps NaN to 0.  `raw + Q_OFFSET` is an i32 sum
+             * (lib.rs:423): where `raw` saturated at i32::MAX -- w / s = +inf, a
+             * tiny non-zero group whose f16 scale rounded to 0 -- a release
+             * build wraps to a negative value, which the clamp turns into code
+             * 0 (a debug build panics there).  The release behaviour is
+             * restated: the sum is formed in 64 bits and wrapped by hand. */
             float q = roundf(weight[(size_t)r * n + col] / s);
             long long raw;
             if (q != q) raw = 0;
@@ -143,6 +147,7 @@ void ko_quantize(const float *weight, int k, int n, int groupsize, int32_t *code
             else if (q <= -2147483648.0f) raw = -2147483648LL;
             else raw = (long long)q;
             long long shifted = raw + 8;
+            if (shifted > 2147483647LL) shifted -= 4294967296LL;
             if (shifted < 0) shifted = 0;
             if (shifted > 15) shifted = 15;
             codes[(size_t)r * n + col] = (int32_t)shifted;

@@ -605,3 +605,62 @@ def test_prefill_positive_mean_activations(oracle, m, k, n):
     x = oracle.np_f32_to_bf16(np.abs(oracle.np_bf16_to_f32(x)))
     b, s = pack.repack_gptq(q, s_bits, None, 128)
     _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
+
+
+# ---------------------------------------------------------------- one scale per column (groupsize -1)
+
+@pytest.mark.parametrize("m", [1, 16, 24, 64, 128, 300, 2048])
+@pytest.mark.parametrize("k,n", [(2560, 8192), (9216, 2560), (4096, 2560)])
+def test_per_column_scales_at_model_shapes(oracle, m, k, n):
+    """groupsize -1 at any K (lib.rs:126-130; the reference's own cases stop at K = 256,
+    parity.rs:213-214): the shipped dispatch, so the unsliced and K-sliced small-M plans, the
+    two-slab instance, the sliced mid-M kernel and the sliced matrix-core kernel all index the one
+    row of scales, and the matrix-core kernel's accumulator carries the offset term over the whole
+    of K without a rescale step in between."""
+    x, q, s_bits = oracle.gen_problem(m, k, n, -1, seed=m + k + n, sigma=0.5 if m > 64 else 1.0)
+    assert s_bits.shape == (1, n)
+    b, s = pack.repack_gptq(q, s_bits, None, -1)
+    _run_case(oracle, m, k, n, -1, x, b, s, q, s_bits)
+
+
+def test_per_column_scales_with_positive_mean_activations(oracle):
+    """|N(0,1)| activations over K = 9216 with one scale per column: the offset the matrix-core
+    kernel removes after the K loop is then at its largest relative to the result."""
+    m, k, n = 2048, 9216, 2560
+    x, q, s_bits = oracle.gen_problem(m, k, n, -1, seed=4242)
+    x = oracle.np_f32_to_bf16(np.abs(oracle.np_bf16_to_f32(x)))
+    b, s = pack.repack_gptq(q, s_bits, None, -1)
+    _run_case(oracle, m, k, n, -1, x, b, s, q, s_bits)
+
+
+@pytest.mark.parametrize("m", [16, 64, 512])
+def test_per_column_scales_with_adapters_and_fused_swiglu(oracle, m):
+    """groupsize -1 through the calls with a low-rank term and through the fused gate+up SwiGLU
+    (K = 2560, the model's MLP input), each against the oracle."""
+    k, n, g = 2560, 2048, -1
+    x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=900 + m, sigma=0.5)
+    b, s = pack.repack_gptq(q, s_bits, None, g)
+    bt, st = upload_packed(b, s)
+    xt = bf16_tensor(x)
+    y_ref = oracle.c_w4a16_cpu_path(x, q, s_bits, g)
+    ranks, scales = (16, 32), (0.5, 1.0)
+    a_list = [oracle.gen_normal_bf16(r, k, 0.05, seed=910 + i) for i, r in enumerate(ranks)]
+    b_list = [oracle.gen_normal_bf16(n, r, 0.05, seed=920 + i) for i, r in enumerate(ranks)]
+    y_lora = y_ref.copy()
+    for a_i, b_i, sc in zip(a_list, b_list, scales):
+        oracle.c_lora_delta_add(y_lora, x, a_i, b_i, sc)
+    y = marlin_gemm.marlin_w4a16_gemm_lora(xt, bt, st, g, bf16_tensor(np.concatenate(a_list, axis=0)),
+                                           bf16_tensor(np.concatenate(b_list, axis=1)), ranks, scales)
+    torch.cuda.synchronize()
+    err, _, _ = row_errors(bf16_bits(y), y_lora, oracle)
+    assert err.max() <= ROW_TOL, err.max()
+    # the same weights as gate, a second set as up
+    _, q_up, s_up = oracle.gen_problem(1, k, n, g, seed=930 + m)
+    b_up, s_up_t = pack.repack_gptq(q_up, s_up, None, g)
+    b_gu, s_gu = pack.interleave_gate_up(b, s, b_up, s_up_t, g)
+    bgt, sgt = upload_packed(b_gu, np.asarray(s_gu).view(np.uint16))
+    h = marlin_gemm.marlin_w4a16_gemm_swiglu(xt, bgt, sgt, g)
+    torch.cuda.synchronize()
+    h_ref = oracle.c_swiglu_f32(y_ref, oracle.c_w4a16_cpu_path(x, q_up, s_up, g))
+    err, _, _ = row_errors(bf16_bits(h), h_ref, oracle)
+    assert err.max() <= ROW_TOL, err.max()

@@ -20,7 +20,7 @@ def test_library_exports_every_declared_symbol():
     raw = ctypes.CDLL(str(_lib.LIB_PATH))
     for name in declared:
         assert hasattr(raw, name), name
-    assert _lib.load().kiln_w4a16_layout_version() == 1
+    assert _lib.load().kiln_w4a16_layout_version() == 2
     assert _lib.status_string(0) == "ok" and "zero-point" in _lib.status_string(5)
 
 
@@ -232,6 +232,9 @@ def test_artifact_round_trip_and_rejections(tmp_path, oracle):
     expect_error(magic, "not a packed-weight artefact")
     version = bytearray(raw); version[8] = 99
     expect_error(version, "layout version 99")
+    # revision 1 interleaved gate and up by 32 columns; a fused pack of that age would be paired wrongly
+    older = bytearray(raw); older[8] = 1
+    expect_error(older, "layout version 1 != library's 2")
     shape = bytearray(raw); shape[16] = 1          # k = 257
     expect_error(shape, "inconsistent artefact header")
     assert L.kiln_w4a16_artifact_read(str(tmp_path / "missing").encode(), b2.ctypes.data, s2.ctypes.data) == _lib.PROJ_ERR
@@ -490,3 +493,28 @@ def test_layer_wiring_keeps_bf16_without_a_gpu_and_reproduces_the_reference_sele
     y = layer.forward(PackKind.KProj, x)
     assert tuple(y.shape) == (2, 3, 256) and torch.equal(y, x @ layer.weights_t[PackKind.KProj])
     assert marlin_proj.shape_is_supported(2560, 1024) and not marlin_proj.shape_is_supported(2560, 32)
+
+
+def test_bf16_drop_switch_follows_the_environment(monkeypatch):
+    """`KILN_DISABLE_MARLIN_BF16_DROP` (forward.rs:1565-1580): install drops the bf16 copy unless the
+    variable says 1 / true / yes; an explicit argument wins over the environment."""
+    import torch
+    from kiln_amd import layer_pack
+    from kiln_amd.layer_pack import LayerProjections, PackKind
+    from kiln_amd.marlin_proj import MarlinPackedProj
+    stand_in = MarlinPackedProj(torch.zeros(8, 512, dtype=torch.int32), torch.zeros(1, 256, dtype=torch.float16), 128, 128, 256)
+
+    def install(**kw):
+        layer = LayerProjections({PackKind.QProj: torch.zeros(128, 256, dtype=torch.bfloat16)})
+        layer_pack.install_packed(layer, PackKind.QProj, stand_in, **kw)
+        assert layer.is_packed(PackKind.QProj)
+        return layer.weights_t[PackKind.QProj] is None
+
+    monkeypatch.delenv("KILN_DISABLE_MARLIN_BF16_DROP", raising=False)
+    assert not marlin_proj.bf16_drop_disabled() and install() is True
+    for v, disabled in [("1", True), ("TRUE", True), (" yes ", True), ("0", False), ("on", False), ("", False)]:
+        monkeypatch.setenv("KILN_DISABLE_MARLIN_BF16_DROP", v)
+        assert marlin_proj.bf16_drop_disabled() is disabled
+        assert install() is (not disabled)
+    monkeypatch.setenv("KILN_DISABLE_MARLIN_BF16_DROP", "1")
+    assert install(drop_bf16=True) is True

@@ -168,6 +168,31 @@ def test_quantizer_ties_clamp_and_zero_group(oracle):
         assert np.all(codes[:, 1] == 8) and np.all(deq[:, 1] == 0.0)
 
 
+def test_quantizer_where_the_scale_rounds_to_zero_or_infinity(oracle):
+    """Worked by hand from lib.rs:405-427.  A group of magnitude 1e-30: s = f16(1.3e-31) = 0, so w / s is
+    +inf, -inf or (0 / 0) NaN; `as i32` gives i32::MAX, i32::MIN, 0; `raw + 8` is an i32 sum -- i32::MAX + 8
+    wraps to a negative value in a release build (a debug build panics), the clamp makes it code 0; MIN + 8
+    clamps to 0; NaN gives 8.  Dequantised values are (code - 8) * 0.  A group of magnitude 3e38: s = f16
+    infinity, w / inf = 0, code 8, dequant 0 * inf = NaN."""
+    k, n = 128, 256
+    w = np.zeros((k, n), dtype=np.float32)
+    w[:4, 0] = [1e-30, -1e-30, 0.0, 5e-31]
+    w[:3, 1] = [3e38, -3e38, 1.0]
+    for fn in (oracle.c_quantize, oracle.np_quantize):
+        with np.errstate(all="ignore"):
+            codes, scales, deq = fn(w, 128)
+        assert scales[0, 0] == 0x0000 and scales[0, 1] == 0x7C00
+        assert list(codes[:4, 0]) == [0, 0, 8, 0]
+        assert np.all(deq[:4, 0] == 0.0)
+        assert list(codes[:3, 1]) == [8, 8, 8] and np.all(np.isnan(deq[:3, 1]))
+    from kiln_amd.marlin_gemm import pack
+    with np.errstate(all="ignore"):
+        b, s, deq = pack.quantize_and_pack(w, k, n, 128)          # the product's host quantiser: the same codes
+    q, _ = pack.unpack_to_gptq(b, s, 128)
+    got = oracle.np_unpack_gptq(q.view(np.uint32))
+    assert list(got[:4, 0]) == [0, 0, 8, 0] and list(got[:3, 1]) == [8, 8, 8]
+
+
 @pytest.mark.parametrize("groupsize", [128, -1])
 def test_quantizer_invariants_and_c_vs_numpy(oracle, groupsize):
     k, n = 256, 256

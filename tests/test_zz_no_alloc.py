@@ -69,3 +69,54 @@ def test_static_scratch_entry_point_refuses_what_does_not_fit():
     assert L.kiln_marlin_w4a16_gemm_static_scratch(p, p, p, p, 16, 200, 9216, 128, dev, stream) == _lib.ERR_PROB_SHAPE
     assert L.kiln_marlin_w4a16_gemm_static_scratch(p, p, p, p, 0, 2560, 9216, 128, dev, stream) == _lib.OK
     torch.cuda.synchronize()
+
+
+def test_static_scratch_calls_allocate_nothing_and_replay_from_a_graph(oracle):
+    """What the entry point is for: device memory in use is the same before and after a run of calls, and
+    after one eager call per shape on the device (the library's one-time queries: the array's address,
+    the kernels' LDS limits) the calls can be captured into a graph and replayed."""
+    L = _lib.load()
+    g = 128
+    shapes = [(16, 9216, 2560), (4, 2560, 8192)]
+    problems = []
+    for m, k, n in shapes:
+        x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=m + n)
+        b, s = pack.repack_gptq(q, s_bits, None, g)
+        bt, st = upload_packed(b, s)
+        problems.append((m, k, n, bf16_tensor(x), bt, st, torch.empty((m, n), dtype=torch.bfloat16, device="cuda")))
+    stream = torch.cuda.Stream()
+    dev = torch.cuda.current_device()
+
+    def calls():
+        for m, k, n, xt, bt, st, out in problems:
+            rc = L.kiln_marlin_w4a16_gemm_static_scratch(xt.data_ptr(), bt.data_ptr(), out.data_ptr(), st.data_ptr(),
+                                                         m, n, k, g, dev, stream.cuda_stream)
+            assert rc == _lib.OK
+
+    with torch.cuda.stream(stream):
+        for _ in range(60):                         # eager warm-up (also of the runtime's own launch pools)
+            calls()
+        stream.synchronize()
+        eager = [p[6].clone() for p in problems]
+        free_before = torch.cuda.mem_get_info()[0]
+        for _ in range(50):
+            calls()
+        stream.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            calls()
+        for replay in range(4):
+            for p in problems:
+                p[6].fill_(float("nan"))
+            graph.replay()
+            stream.synchronize()
+            for p, e in zip(problems, eager):
+                assert torch.equal(p[6].view(torch.int16), e.view(torch.int16)), f"replay {replay}"
+            calls()                                 # eager work between replays
+            stream.synchronize()
+    # nothing gave up on the way: the array's sticky word reads zero
+    word = ctypes.c_uint32(0xFFFFFFFF)
+    assert L.kiln_w4a16_workspace_check(None, ctypes.byref(word), None) == _lib.OK
+    torch.cuda.synchronize()
+    assert word.value == 0
