@@ -216,6 +216,25 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu_lora(
     int n_adapters, const int *ranks, const float *scales);
 
 /*
+ * y[m, n_down] = down( silu(gate(x)) * up(x) ): the MLP of a layer as one call, at any m.  The reference's
+ * swiglu_ffn_impl (crates/kiln-model/src/forward.rs:2723-2848) issues the gate GEMM, the up GEMM, silu, the
+ * multiply and the down GEMM one after the other; this is kiln_w4a16_gemm_swiglu followed by
+ * kiln_marlin_w4a16_gemm -- two launches -- with silu(gate) * up kept in the workspace, rounded to bf16 once.
+ *   x                    bf16 [m, hidden]
+ *   b_gate_up, s_gate_up packed for 2 * n_out columns by kiln_w4a16_interleave_gate_up(_device); n_out % 128 == 0
+ *   b_down, s_down       the down projection [n_out, n_down], packed as for kiln_marlin_w4a16_gemm
+ *   y                    bf16 [m, n_down]
+ *   workspace            kiln_w4a16_mlp_workspace_bytes(m, hidden, n_out, n_down) bytes (never decreases with m),
+ *                        zeroed prefix as for every entry point
+ */
+kiln_marlin_status_t kiln_w4a16_mlp(
+    const void *x, const void *b_gate_up, const void *s_gate_up, const void *b_down, const void *s_down,
+    void *y, int prob_m, int hidden, int n_out, int n_down,
+    void *workspace, int groupsize, int dev, void *stream);
+
+size_t kiln_w4a16_mlp_workspace_bytes(int prob_m, int hidden, int n_out, int n_down);
+
+/*
  * out[k, n] (f32, row-major) = (code - 8) * f32(scale), read from the tile
  * layout on the device.  The device-side statement of lib.rs:425; used to
  * prove the repack bit-exact.  No counterpart entry point in the reference.

@@ -24,6 +24,8 @@ EXPORTS = (
     "kiln_w4a16_gemm_swiglu",
     "kiln_w4a16_swiglu_workspace_bytes",
     "kiln_w4a16_gemm_swiglu_lora",
+    "kiln_w4a16_mlp",
+    "kiln_w4a16_mlp_workspace_bytes",
     "kiln_w4a16_quantize_and_pack_device",
     "kiln_w4a16_interleave_gate_up_device",
     "kiln_w4a16_repack_gptq_device",
@@ -166,6 +168,10 @@ def _load(tuning: bool) -> ctypes.CDLL:
     L.kiln_w4a16_gemm_swiglu.argtypes = [vp, vp, vp, vp, i, i, i, vp, i, i, vp]
     L.kiln_w4a16_gemm_swiglu_lora.restype = i
     L.kiln_w4a16_gemm_swiglu_lora.argtypes = L.kiln_w4a16_gemm_lora.argtypes
+    L.kiln_w4a16_mlp.restype = i
+    L.kiln_w4a16_mlp.argtypes = [vp, vp, vp, vp, vp, vp, i, i, i, i, vp, i, i, vp]
+    L.kiln_w4a16_mlp_workspace_bytes.restype = c.c_size_t
+    L.kiln_w4a16_mlp_workspace_bytes.argtypes = [i, i, i, i]
     L.kiln_w4a16_quantize_and_pack_device.restype = i
     L.kiln_w4a16_quantize_and_pack_device.argtypes = [vp, i, i, i, vp, vp, i, vp]
     L.kiln_w4a16_repack_gptq_device.restype = i

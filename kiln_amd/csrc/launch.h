@@ -21,6 +21,7 @@ constexpr size_t kWsCounterCapacity = kWsErrorOffset;  // bytes of the counter r
 constexpr size_t kWsFlaggedBytes = 4 * 1024 * 1024;
 constexpr size_t kWsFoldFlagBytes = 16 * 4096;
 constexpr size_t kWsFoldFlagOffset = kWsCounterBytes + kWsFlaggedBytes - kWsFoldFlagBytes;
+constexpr size_t kWsZeroedBytes = kWsCounterBytes + kWsFlaggedBytes;
 enum WaitGaveUp : unsigned {
     kGaveUpDecodeExchange = 1u,  // K slices of a launch of up to 16 rows
     kGaveUpMidExchange = 2u,     // K slices of a launch of 33...192 rows

@@ -19,7 +19,7 @@ constexpr int kMaxDevices = 16;
 constexpr size_t kCounterBytes = kWsCounterBytes;
 constexpr size_t kCounterCapacity = kWsCounterCapacity;  // what counters may use of it
 constexpr size_t kFlaggedBytes = kWsFlaggedBytes;
-constexpr size_t kZeroedBytes = kCounterBytes + kFlaggedBytes;
+constexpr size_t kZeroedBytes = kWsZeroedBytes;
 constexpr size_t kFoldFlagBytes = kWsFoldFlagBytes;
 constexpr size_t kFoldFlagOffset = kWsFoldFlagOffset;
 
@@ -1137,6 +1137,37 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu_lora(const void *A, const void *B, v
     // follow the packed columns, so an adapter of gate and one of up are two column blocks of one stacked B
     const LoraSpec lora{lora_a, lora_b, r_total, n_adapters, ranks, scales};
     return gemm_any(A, B, C, s, prob_m, 2 * n_out, prob_k, workspace, groupsize, dev, stream, -1, -1, -1, &lora, true);
+}
+
+// ---- the MLP of a layer as one call -------------------------------------------------------------------
+// workspace: [what the two GEMMs need, the larger of the two] | H = bf16 [m, n_out]
+static size_t mlp_h_offset(int m, int k1, int n_out, int n2) {
+    const size_t a = kiln_w4a16_swiglu_workspace_bytes(m, n_out, k1), b = kiln_w4a16_workspace_bytes(m, n2, n_out);
+    return ((a > b ? a : b) + 255) & ~(size_t)255;
+}
+
+size_t kiln_w4a16_mlp_workspace_bytes(int prob_m, int hidden, int n_out, int n_down) {
+    if (prob_m < 1) prob_m = 1;
+    if (hidden <= 0 || n_out <= 0 || n_down <= 0 || n_out > INT32_MAX / 2) return kZeroedBytes;
+    return mlp_h_offset(prob_m, hidden, n_out, n_down) + (size_t)prob_m * n_out * 2;
+}
+
+kiln_marlin_status_t kiln_w4a16_mlp(const void *x, const void *b_gate_up, const void *s_gate_up, const void *b_down,
+                                    const void *s_down, void *y, int prob_m, int hidden, int n_out, int n_down,
+                                    void *workspace, int groupsize, int dev, void *stream) {
+    if (prob_m < 0 || hidden < 0 || n_out < 0 || n_down < 0 || n_out > INT32_MAX / 2) return KILN_W4A16_ERR_PROB_SHAPE;
+    if (!shape_ok(2 * n_out, hidden, groupsize) || !shape_ok(n_down, n_out, groupsize)) return KILN_W4A16_ERR_PROB_SHAPE;
+    if (prob_m == 0 || hidden == 0 || n_out == 0 || n_down == 0) return KILN_W4A16_OK;
+    if (!x || !b_gate_up || !s_gate_up || !b_down || !s_down || !y || !workspace) return KILN_W4A16_ERR_ARGUMENT;
+    char *ws = reinterpret_cast<char *>(workspace);
+    void *h = ws + mlp_h_offset(prob_m, hidden, n_out, n_down);
+    // Two launches with H in between.  (One launch for both -- down blocks resident from the start, their weights
+    // in registers, waiting for their columns of H -- measured level with the two, 15.2 us at 16 rows: every hop
+    // of the hand-over inside a launch crosses the dies' memory system, about a microsecond each.)
+    const kiln_marlin_status_t st = gemm_any(x, b_gate_up, h, s_gate_up, prob_m, 2 * n_out, hidden, workspace, groupsize, dev,
+                                             stream, -1, -1, -1, nullptr, true);
+    if (st != KILN_W4A16_OK) return st;
+    return gemm_any(h, b_down, y, s_down, prob_m, n_down, n_out, workspace, groupsize, dev, stream, -1, -1, -1, nullptr);
 }
 
 size_t kiln_w4a16_swiglu_workspace_bytes(int prob_m, int n_out, int prob_k) {

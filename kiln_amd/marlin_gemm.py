@@ -359,6 +359,38 @@ def marlin_w4a16_gemm_swiglu(a: torch.Tensor, b_packed: torch.Tensor, scales: to
     return out
 
 
+def marlin_w4a16_mlp(x: torch.Tensor, b_gate_up: torch.Tensor, s_gate_up: torch.Tensor, b_down: torch.Tensor,
+                     s_down: torch.Tensor, groupsize: int, *, out: torch.Tensor | None = None) -> torch.Tensor:
+    """`down(silu(gate(x)) * up(x))`: `[m, hidden]` bf16 -> `[m, n_down]` bf16, the whole MLP of a layer
+    (crates/kiln-model/src/forward.rs:2723-2848) as one call: the fused gate+up SwiGLU GEMM, then the down
+    GEMM, `silu(gate) * up` kept in the workspace between them.
+    `b_gate_up` / `s_gate_up` from `pack.interleave_gate_up`, `b_down` / `s_down` the packed down projection."""
+    m, k, n = _check_gemm_args(x, b_gate_up, s_gate_up, groupsize)
+    if n % 256 != 0:
+        _bail(f"fused gate+up width {n} must be a multiple of 256")
+    n_out = n // 2
+    if b_down.dim() != 2 or s_down.dim() != 2 or b_down.shape[0] * 16 != n_out:
+        _bail(f"down projection must be packed for k = {n_out} (b_down is {tuple(b_down.shape)})")
+    _, _, n_down = _check_gemm_args(torch.empty((0, n_out), dtype=torch.bfloat16, device=x.device), b_down, s_down, groupsize)
+    lib = _lib.load()
+    x, b_gate_up, s_gate_up = x.contiguous(), b_gate_up.contiguous(), s_gate_up.contiguous()
+    b_down, s_down = b_down.contiguous(), s_down.contiguous()
+    if out is None:
+        out = torch.empty((m, n_down), dtype=torch.bfloat16, device=x.device)
+    if m == 0:
+        return out
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
+        ws = _workspace(x.device, stream, lib.kiln_w4a16_mlp_workspace_bytes(m, k, n_out, n_down))
+        status = lib.kiln_w4a16_mlp(x.data_ptr(), b_gate_up.data_ptr(), s_gate_up.data_ptr(), b_down.data_ptr(),
+                                    s_down.data_ptr(), out.data_ptr(), m, k, n_out, n_down, ws.data_ptr(), groupsize,
+                                    x.device.index or 0, stream)
+    if status != 0:
+        raise MarlinGemmError(f"kiln_w4a16_mlp failed with status {status}: {_lib.status_string(status)} "
+                              f"(m={m}, hidden={k}, n_out={n_out}, n_down={n_down})")
+    return out
+
+
 def marlin_w4a16_gemm_lora(a: torch.Tensor, b_packed: torch.Tensor, scales: torch.Tensor,
                            groupsize: int, lora_a: torch.Tensor, lora_b: torch.Tensor,
                            ranks, lora_scales, *, out: torch.Tensor | None = None) -> torch.Tensor:
