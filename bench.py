@@ -37,7 +37,27 @@ TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median rep
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
 # copy (x1.9989 and x1.0): 12278.6 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
-GATE_UP_M16_TRAFFIC_BYTES = 25722600
+# The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
+# kernel instance on one plan: where the planner picks another for the headline shape the line reports no
+# traffic instead of this one.
+GATE_UP_M16_TRAFFIC = {"bytes": 25722600, "kernel": "w4a16_decode_gmp_kernel<5, 2, 4, false>", "blocks": 231}
+MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
+
+
+def decode_kernel_of_plan(lib, m: int, k: int, n: int, cus: int):
+    """Name and grid of the small-M kernel instance the dispatcher runs for (m, k, n), from the library's
+    own plan query -- (kernel name, blocks)."""
+    import ctypes
+    out = (ctypes.c_int * 8)()
+    if lib.kiln_w4a16_debug_decode_plan(m, n, k, cus, out) != 0:
+        return "unknown", 0
+    ks, gs, u, bps, waves, direct, regs, gm_tiles = list(out)
+    if gm_tiles < 0:        # the private-staging instance: <tiles, groups per wavefront, LDS-direct loads per group, adapters>
+        aq = 1 if m <= 4 else (2 if m <= 8 else 4)
+        return f"w4a16_decode_gmp_kernel<{-gm_tiles}, {-(-gs // waves)}, {aq}, false>", bps * ks
+    if gm_tiles > 0:
+        return f"w4a16_decode_gm_kernel<{gm_tiles}, {-(-gs // waves)}, false>", bps * ks
+    return (f"w4a16_decode_gmr_kernel (run {u})" if regs else f"w4a16_decode_kernel<{u}, {bool(direct)}>"), bps * ks
 
 
 def algorithmic_bytes(m: int, k: int, n: int) -> int:
@@ -161,6 +181,37 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
     extra["decode_layer_m16_four_linears"] = {"us": round(t_p / 64 * 1e6, 2),
                                               "with_two_lora_adapters_per_projection_us": round(t_l / 64 * 1e6, 2)}
     del lw
+
+    # projections that read the same input, as separate launches and packed side by side as one GEMM (the columns
+    # of a GEMM are independent): q | k | v of a full-attention layer, in_proj_qkv | in_proj_z of a GDN layer
+    for name, widths in (("attention_qkv", (8192, 1024, 1024)), ("gdn_in_proj_qkv_z", (8192, 4096))):
+        for m_f in (1, 16):
+            parts = [[make_layer(2560, n_) for _ in range(8)] for n_ in widths]
+            whole = [make_layer(2560, sum(widths)) for _ in range(8)]
+            x_ = torch.randn(m_f, 2560, device=dev).to(torch.bfloat16)
+            po = [torch.empty(m_f, n_, dtype=torch.bfloat16, device=dev) for n_ in widths]
+            wo = torch.empty(m_f, sum(widths), dtype=torch.bfloat16, device=dev)
+            def fn_parts(i):
+                for j in range(len(widths)):
+                    marlin_gemm.marlin_w4a16_gemm(x_, *parts[j][i % 8], GROUP, out=po[j])
+            def fn_whole(i):
+                marlin_gemm.marlin_w4a16_gemm(x_, *whole[i % 8], GROUP, out=wo)
+            t_parts, _ = timed_graph(fn_parts, 64)
+            t_whole, _ = timed_graph(fn_whole, 64)
+            extra[f"{name}_m{m_f}"] = {"separate_launches_us": round(t_parts / 64 * 1e6, 2),
+                                       "one_launch_side_by_side_us": round(t_whole / 64 * 1e6, 2)}
+    # the MLP as one call (fused gate+up SwiGLU, then down: two launches)
+    from kiln_amd.marlin_gemm import marlin_w4a16_mlp
+    mw = [(make_layer(2560, 18432), make_layer(9216, 2560)) for _ in range(8)]
+    for m_f in (1, 16):
+        x_ = torch.randn(m_f, 2560, device=dev).to(torch.bfloat16)
+        o_ = torch.empty(m_f, 2560, dtype=torch.bfloat16, device=dev)
+        def fn_mlp(i):
+            (b1, s1), (b2, s2) = mw[i % 8]
+            marlin_w4a16_mlp(x_, b1, s1, b2, s2, GROUP, out=o_)
+        t_mlp, _ = timed_graph(fn_mlp, 64)
+        extra[f"mlp_m{m_f}_one_call_two_launches"] = {"us": round(t_mlp / 64 * 1e6, 2)}
+    del mw
 
     # per-launch distribution and wrapper-inclusive cost of the headline GEMM (eager launches)
     ws_ = [make_layer(2560, 18432) for _ in range(16)]
@@ -286,6 +337,11 @@ def main() -> int:
         dst = torch.empty_like(src)
         dst.copy_(src)                                  # reads 64 MiB, writes 64 MiB
         if args.profile == "decode":
+            from kiln_amd import _lib
+            cus = torch.cuda.get_device_properties(dev).multi_processor_count
+            for name, kn in shapes.items():     # which instances the counters of this run belong to
+                print(f"bench.py --profile decode: {name} M={M} runs %s x %d blocks" % decode_kernel_of_plan(_lib.load(), M, *kn, cus),
+                      file=sys.stderr)
             for i in range(args.steps):
                 step(i)
         elif args.profile == "decode_m1":
@@ -349,10 +405,11 @@ def main() -> int:
     replay_log = {}
 
     def timed_graph(fn, count, tag=None):
-        """Capture `count` calls of fn(i) into one graph; replay once untimed, then TIMED_REPLAYS times,
-        each replay timed on its own between two synchronisations (HIP events on the launch stream around
-        exactly `count` calls); returns the median replay (replay to replay the same graph reads +-3 %,
-        the first ones after a change of workload high)."""
+        """Capture `count` calls of fn(i) into one graph; replay it untimed, then take TIMED_REPLAYS timed
+        regions, each one replay between two synchronisations with HIP events on the launch stream.  Where
+        `count` calls are shorter than MIN_TIMED_REGION_S the timed graph holds them several times over
+        (whole passes of exactly `count` calls, back to back); returns the median region's time per pass
+        (region to region the same graph reads +-3 %, the first ones after a change of workload high)."""
         g = torch.cuda.CUDAGraph()
         with torch.cuda.stream(stream):
             for i in range(min(count, LAYERS)):
@@ -363,20 +420,38 @@ def main() -> int:
                     fn(i)
             g.replay()
             stream.synchronize()
-            runs = []
-            for _ in range(TIMED_REPLAYS):
+
+            def one_region(graph):
                 e0 = torch.cuda.Event(enable_timing=True)
                 e1 = torch.cuda.Event(enable_timing=True)
                 torch.cuda.synchronize()
                 t0 = time.perf_counter()
                 e0.record(stream)
-                g.replay()
+                graph.replay()
                 e1.record(stream)
                 torch.cuda.synchronize()
-                runs.append((e0.elapsed_time(e1) * 1e-3, time.perf_counter() - t0))
+                return e0.elapsed_time(e1) * 1e-3, time.perf_counter() - t0
+
+            # sizing pass, not reported: a region shorter than MIN_TIMED_REGION_S (K = 20 steps of 15 us are
+            # 0.3 ms: the clocks have not settled and the events' own cost shows) is stretched to it by a graph
+            # that holds the same K calls `reps` times over, back to back, with nothing between them
+            t_ev, _ = one_region(g)
+            reps = max(1, min(4000 // max(count, 1), int(MIN_TIMED_REGION_S / max(t_ev, 1e-6)) + 1))
+            if reps > 1:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g, stream=stream):
+                    for i in range(reps * count):
+                        fn(i)
+                g.replay()
+                stream.synchronize()
+            runs = []
+            for _ in range(TIMED_REPLAYS):
+                t_ev, t_wall = one_region(g)
+                runs.append((t_ev / reps, t_wall / reps))
         runs.sort()
         if tag:
             replay_log[tag] = [round(t / count * 1e6, 3) for t, _ in runs]
+            replay_log[tag.replace("_us_per_replay_sorted", "") + "_passes_of_k_calls_per_timed_region"] = reps
         return runs[len(runs) // 2]
 
     t_step, wall_step = timed_graph(step, args.steps, tag="step_us_per_replay_sorted")
@@ -463,6 +538,10 @@ def main() -> int:
                                   f"{t_deq * 1e3:.1f} ms, matmul {t_mm * 1e3:.1f} ms; "
                                   f"cfg 0 (M=1, 2560x2560) {t_cfg0 * 1e6:.0f} us per pass"}
 
+    from kiln_amd import _lib
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    gu_kernel, gu_blocks = decode_kernel_of_plan(_lib.load(), M, *shapes["gate_up"], cus)
+    traffic_known = (gu_kernel, gu_blocks) == (GATE_UP_M16_TRAFFIC["kernel"], GATE_UP_M16_TRAFFIC["blocks"])
     result = {
         "metric": "w4a16_gemm_decode_effective_bandwidth_m16",
         "value": round(value, 2),
@@ -483,8 +562,9 @@ def main() -> int:
                    "timed_replays": TIMED_REPLAYS, "statistic": "median replay",
                    "wall_ms_per_step": round(wall_step / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": GATE_UP_M16_TRAFFIC_BYTES,
-                     "kernel": "w4a16_decode_gmp_kernel<5, 2, 4, false> (gate+up, M=16, K=2560, N=18432)",
+                     "frac": round(achieved / HBM_PEAK_GBPS, 4),
+                     "traffic": GATE_UP_M16_TRAFFIC["bytes"] if traffic_known else None,
+                     "kernel": f"{gu_kernel} x {gu_blocks} blocks (gate+up, M=16, K=2560, N=18432)",
                      "us_per_launch": round(us_gu, 3), "algorithmic_bytes_per_launch": bytes_gu},
         "cpu_baseline": cpu_baseline,
         "extra": {**extra, **replay_log},

@@ -29,7 +29,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import torch
 
 from . import marlin_gemm, marlin_proj
-from .lora import proj_forward, swiglu_forward, swiglu_lora_fits
+from .lora import fuse_column_blocks, proj_forward, swiglu_forward, swiglu_lora_fits
 from .marlin_proj import MarlinPackedProj, MarlinProjError
 
 
@@ -52,6 +52,11 @@ class PackKind(Enum):
 FULL_ATTENTION_KINDS = (PackKind.QProj, PackKind.KProj, PackKind.VProj, PackKind.OProj)
 LINEAR_ATTENTION_KINDS = (PackKind.InProjQkv, PackKind.InProjZ, PackKind.OutProj, PackKind.InProjA, PackKind.InProjB)
 MLP_KINDS = (PackKind.GateProj, PackKind.UpProj, PackKind.DownProj)
+# Projections of a layer that read the same input: packed side by side they are one GEMM -- the columns of a
+# GEMM are independent of each other -- and one launch instead of three or two per decode step
+# (the reference calls them one after the other: forward.rs:372 `full_attn_qkv_proj_decode_if`, and the GDN
+# block's in-projections).  A launch of this size costs 3...5 us whatever its width.
+SAME_INPUT_GROUPS = ((PackKind.QProj, PackKind.KProj, PackKind.VProj), (PackKind.InProjQkv, PackKind.InProjZ))
 # what the reference itself queues (forward.rs:1884-1890, 2002-2018)
 REFERENCE_KINDS = (PackKind.QProj, PackKind.GateProj, PackKind.UpProj, PackKind.DownProj)
 
@@ -70,6 +75,7 @@ class LayerProjections:
     weights_t: Dict[PackKind, Optional[torch.Tensor]]
     packed: Dict[PackKind, MarlinPackedProj] = field(default_factory=dict)
     gate_up_fused: Optional[MarlinPackedProj] = None   # gate and up interleaved for the SwiGLU entry point
+    same_input_fused: Dict[Tuple[PackKind, ...], MarlinPackedProj] = field(default_factory=dict)   # see SAME_INPUT_GROUPS
 
     def is_packed(self, kind: PackKind) -> bool:
         return kind in self.packed
@@ -87,6 +93,32 @@ class LayerProjections:
         if lora is not None:                                  # unfused, as the reference's bf16 branch
             y = y + ((x @ lora.a.t().to(x.dtype)) @ lora.b.t().to(x.dtype)) * lora_scale
         return y
+
+    def forward_same_input(self, kinds: Sequence[PackKind], x: torch.Tensor, loras: Optional[Dict[PackKind, object]] = None,
+                           lora_scale: float = 1.0) -> Tuple[torch.Tensor, ...]:
+        """The projections `kinds` of one input: one launch on their side-by-side pack where `pack_layers`
+        built it (the results are column ranges of one output tensor), else one `forward` each.  `loras`
+        maps a kind to its adapter(s); on the fused pack they become one stacked set whose projection of x
+        is computed once for all members (stacked rank <= 64 and <= 8 adapters, else the members run
+        one by one)."""
+        kinds = tuple(kinds)
+        loras = loras or {}
+        fused = self.same_input_fused.get(kinds)
+        stacked = None
+        if fused is not None and any(loras.get(k) is not None for k in kinds):
+            widths = [self.packed[k].n for k in kinds]
+            stacked = fuse_column_blocks([loras.get(k) for k in kinds], widths, lora_scale)
+            if sum(stacked.ranks) > 64 or len(stacked.ranks) > 8:
+                fused = None
+        if fused is None:
+            return tuple(self.forward(k, x, loras.get(k), lora_scale) for k in kinds)
+        y = proj_forward(x, fused, stacked)
+        outs, col = [], 0
+        for k in kinds:
+            n = self.packed[k].n
+            outs.append(y[..., col:col + n])
+            col += n
+        return tuple(outs)
 
     def swiglu(self, x: torch.Tensor, gate_lora=None, up_lora=None, lora_scale: float = 1.0) -> torch.Tensor:
         """`silu(gate_proj(x)) * up_proj(x)`, each projection with its LoRA delta (forward.rs:2771-2819):
@@ -125,13 +157,36 @@ def install_packed(layer: LayerProjections, kind: PackKind, packed: MarlinPacked
         layer.weights_t[kind] = None
 
 
+def fuse_same_input(layer: LayerProjections) -> int:
+    """Pack the members of every group of SAME_INPUT_GROUPS that the layer has packed (same k, same
+    groupsize) side by side as one projection.  In the tile layout a packed weight is a sequence of column
+    tiles, each with all of its K, and so are its scales: side by side is one after the other."""
+    built = 0
+    for kinds in SAME_INPUT_GROUPS:
+        members = [layer.packed.get(k) for k in kinds]
+        if any(p is None for p in members):
+            continue
+        k, g = members[0].k, members[0].groupsize
+        if any(p.k != k or p.groupsize != g for p in members):
+            continue
+        n = sum(p.n for p in members)
+        b = torch.cat([p.b_packed.reshape(-1) for p in members]).reshape(k // 16, 2 * n)
+        s = torch.cat([p.scales.reshape(-1) for p in members]).reshape(-1, n)
+        layer.same_input_fused[tuple(kinds)] = MarlinPackedProj(b, s, g, k, n)
+        built += 1
+    return built
+
+
 def pack_layers(layers: Sequence[LayerProjections], kinds: Optional[Sequence[PackKind]] = None,
-                groupsize: int = 128, drop_bf16: Optional[bool] = None, fuse_gate_up: bool = False) -> Dict[str, int]:
+                groupsize: int = 128, drop_bf16: Optional[bool] = None, fuse_gate_up: bool = False,
+                fuse_same_input_groups: bool = False) -> Dict[str, int]:
     """The post-loop batch pack and install (forward.rs:2040-2085): every queued projection goes
     through `pack_from_bf16_batch` (serial copies, threaded host pack); a projection whose shape the
     kernels do not take (`shape_is_supported`, e.g. the 32-column `in_proj_a` / `in_proj_b`) comes
     back as None and keeps its bf16 weight.  With `fuse_gate_up`, gate and up of a layer are also
-    interleaved into one pack for the SwiGLU entry point.  Returns counts for the caller's log line."""
+    interleaved into one pack for the SwiGLU entry point; with `fuse_same_input_groups`, q/k/v and the GDN
+    block's two wide in-projections are also packed side by side as one projection each
+    (`forward_same_input`).  Returns counts for the caller's log line."""
     inputs: List[Tuple[torch.Tensor, int]] = []
     meta: List[PackEntry] = []
     for i, layer in enumerate(layers):
@@ -153,4 +208,7 @@ def pack_layers(layers: Sequence[LayerProjections], kinds: Optional[Sequence[Pac
             b_gu, s_gu = marlin_gemm.interleave_gate_up_device(g.b_packed, g.scales, u.b_packed, u.scales, g.groupsize)
             layer.gate_up_fused = MarlinPackedProj(b_gu, s_gu, g.groupsize, g.k, 2 * g.n)
             n_fused += 1
-    return {"inputs": len(inputs), "packed": n_packed, "kept_bf16": len(inputs) - n_packed, "gate_up_fused": n_fused}
+    stats = {"inputs": len(inputs), "packed": n_packed, "kept_bf16": len(inputs) - n_packed, "gate_up_fused": n_fused}
+    if fuse_same_input_groups:
+        stats["same_input_fused"] = sum(fuse_same_input(layer) for layer in layers)
+    return stats

@@ -99,6 +99,33 @@ def swiglu_forward(x: torch.Tensor, gate_up: MarlinPackedProj, gate_lora=None, u
     return h.reshape(*x.shape[:-1], n_out)
 
 
+def fuse_column_blocks(loras: Sequence, widths: Sequence[int], lora_scale: float = 1.0) -> Optional[StackedLora]:
+    """The adapters of projections that share their input and were packed side by side as one GEMM of
+    `sum(widths)` columns (projection i owns the next `widths[i]` columns): one stacked set for that GEMM.
+    The A matrices are row-concatenated as they are -- they all read the same x, so one projection of x
+    onto the stacked rank axis serves every member -- and B becomes block-structured: projection i's B
+    entries sit in its own rows and its own adapters' rank columns, zeros elsewhere.  `loras[i]` is None,
+    a LoraProjectionWeights (scaled by `lora_scale`) or a StackedLora.  None if no member has an adapter."""
+    sides = [_as_stacked(l, lora_scale) for l in loras]
+    if all(s is None for s in sides):
+        return None
+    r_total = sum(sum(s.ranks) for s in sides if s is not None)
+    ref = next(s for s in sides if s is not None)
+    b_cat = torch.zeros((sum(widths), r_total), dtype=torch.bfloat16, device=ref.b_cat.device)
+    row = col = 0
+    for s, width in zip(sides, widths):
+        if s is not None:
+            if s.b_cat.shape[0] != width:
+                raise MarlinProjError(f"fuse_column_blocks: adapter B has {s.b_cat.shape[0]} rows, its projection {width} columns")
+            r = sum(s.ranks)
+            b_cat[row:row + width, col:col + r] = s.b_cat
+            col += r
+        row += width
+    present = [s for s in sides if s is not None]
+    return StackedLora(torch.cat([s.a_cat for s in present], dim=0).contiguous(), b_cat,
+                       tuple(r for s in present for r in s.ranks), tuple(v for s in present for v in s.scales))
+
+
 def swiglu_lora_fits(gate_lora, up_lora) -> bool:
     """Can `swiglu_forward` take these adapters (stacked rank <= 64, <= 8 adapters)?"""
     ranks = []

@@ -371,7 +371,12 @@ def marlin_w4a16_mlp(x: torch.Tensor, b_gate_up: torch.Tensor, s_gate_up: torch.
     n_out = n // 2
     if b_down.dim() != 2 or s_down.dim() != 2 or b_down.shape[0] * 16 != n_out:
         _bail(f"down projection must be packed for k = {n_out} (b_down is {tuple(b_down.shape)})")
-    _, _, n_down = _check_gemm_args(torch.empty((0, n_out), dtype=torch.bfloat16, device=x.device), b_down, s_down, groupsize)
+    n_down = s_down.shape[1]
+    groups = 1 if groupsize == -1 else n_out // 128
+    if n_down % 256 != 0 or b_down.shape[1] != 2 * n_down or s_down.shape[0] != groups:
+        _bail(f"down projection: b_down {tuple(b_down.shape)} / s_down {tuple(s_down.shape)} do not match k = {n_out}")
+    if b_down.dtype != torch.int32 or s_down.dtype != torch.float16 or not (b_down.is_cuda and s_down.is_cuda):
+        _bail("down projection: b_down must be int32 and s_down float16, both on CUDA")
     lib = _lib.load()
     x, b_gate_up, s_gate_up = x.contiguous(), b_gate_up.contiguous(), s_gate_up.contiguous()
     b_down, s_down = b_down.contiguous(), s_down.contiguous()

@@ -136,3 +136,67 @@ def test_fused_gate_up_swiglu_of_a_layer_with_adapters(oracle, packed_layers):
     oracle.c_lora_delta_add(gate1, x, a0, b0, 0.5)
     err1, _, _ = row_errors(bf16_bits(h1), oracle.c_swiglu_f32(gate1, up_plain), oracle)
     assert err1.max() <= 1e-2
+
+
+@pytest.fixture(scope="module")
+def fused_layers(oracle):
+    h0, d0 = _weights(oracle, FULL, 1)
+    h1, d1 = _weights(oracle, LINEAR, 2)
+    layers = [LayerProjections(d0), LayerProjections(d1)]
+    stats = layer_pack.pack_layers(layers, fuse_same_input_groups=True)
+    return layers, [h0, h1], stats
+
+
+@pytest.mark.parametrize("m", [1, 16, 40, 300])
+@pytest.mark.parametrize("layer_idx,kinds", [(0, (PackKind.QProj, PackKind.KProj, PackKind.VProj)),
+                                             (1, (PackKind.InProjQkv, PackKind.InProjZ))])
+def test_projections_of_one_input_as_one_gemm(oracle, fused_layers, layer_idx, kinds, m):
+    """q | k | v (2560 -> 8192 + 1024 + 1024) and in_proj_qkv | in_proj_z (2560 -> 8192 + 4096) packed side by
+    side: one launch, the members' results are column ranges of its output; each against the oracle and
+    against the member's own launch."""
+    layers, host, stats = fused_layers
+    assert stats["same_input_fused"] == 2 and tuple(kinds) in layers[layer_idx].same_input_fused
+    layer = layers[layer_idx]
+    fused = layer.same_input_fused[tuple(kinds)]
+    assert fused.n == sum(host[layer_idx][k].shape[1] for k in kinds) and tuple(fused.b_packed.shape) == (HIDDEN // 16, 2 * fused.n)
+    x = oracle.gen_normal_bf16(m, HIDDEN, 0.5 if m > 64 else 1.0, seed=m + layer_idx)
+    xt = bf16_tensor(x)
+    outs = layer.forward_same_input(kinds, xt)
+    torch.cuda.synchronize()
+    for kind, y in zip(kinds, outs):
+        codes, s_bits, _ = oracle.c_quantize(host[layer_idx][kind], 128)
+        y_ref = oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128)
+        assert tuple(y.shape) == y_ref.shape
+        err, yv, _ = row_errors(bf16_bits(y), y_ref, oracle)
+        assert np.all(np.isfinite(yv)) and err.max() <= 1e-2, (kind, m, err.max())
+        alone = layer.forward(kind, xt).float()
+        assert torch.all((y.float() - alone).abs() <= 1e-2 * alone.abs().amax(dim=1, keepdim=True))
+    # rank-3 input, as the callers pass it (marlin_proj.rs:285-319)
+    outs3 = layer.forward_same_input(kinds, xt.reshape(1, m, HIDDEN))
+    assert all(tuple(o.shape) == (1, m, host[layer_idx][k].shape[1]) for o, k in zip(outs3, kinds))
+
+
+@pytest.mark.parametrize("m", [4, 16, 48])
+def test_projections_of_one_input_with_adapters(oracle, fused_layers, m):
+    """Adapters on q_proj (two, stacked) and v_proj (one), none on k_proj: on the side-by-side pack they are
+    one stacked set -- A matrices row-concatenated, B block-structured -- and x is projected once."""
+    from kiln_amd.lora import LoraProjectionWeights, stack_adapters
+    layers, host, _ = fused_layers
+    kinds = (PackKind.QProj, PackKind.KProj, PackKind.VProj)
+    x = oracle.gen_normal_bf16(m, HIDDEN, 1.0, seed=70 + m)
+    spec = {PackKind.QProj: ((16, 8), (0.5, 2.0)), PackKind.VProj: ((16,), (1.0,))}
+    raw, loras = {}, {}
+    for j, (kind, (ranks, scales)) in enumerate(spec.items()):
+        n = host[0][kind].shape[1]
+        raw[kind] = [(oracle.gen_normal_bf16(r, HIDDEN, 0.05, 100 + 10 * j + i), oracle.gen_normal_bf16(n, r, 0.05, 200 + 10 * j + i))
+                     for i, r in enumerate(ranks)]
+        loras[kind] = stack_adapters([LoraProjectionWeights(bf16_tensor(a), bf16_tensor(b)) for a, b in raw[kind]], scales)
+    outs = layers[0].forward_same_input(kinds, bf16_tensor(x), loras)
+    torch.cuda.synchronize()
+    for kind, y in zip(kinds, outs):
+        codes, s_bits, _ = oracle.c_quantize(host[0][kind], 128)
+        y_ref = oracle.c_w4a16_cpu_path(x, oracle.np_pack_gptq(codes), s_bits, 128)
+        for (a_i, b_i), sc in zip(raw.get(kind, []), spec.get(kind, ((), ()))[1]):
+            oracle.c_lora_delta_add(y_ref, x, a_i, b_i, sc)
+        err, _, _ = row_errors(bf16_bits(y), y_ref, oracle)
+        assert err.max() <= 1e-2, (kind, m, err.max())

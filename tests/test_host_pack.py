@@ -518,3 +518,27 @@ def test_bf16_drop_switch_follows_the_environment(monkeypatch):
         assert install() is (not disabled)
     monkeypatch.setenv("KILN_DISABLE_MARLIN_BF16_DROP", "1")
     assert install(drop_bf16=True) is True
+
+
+def test_adapters_of_side_by_side_projections_become_one_block_structured_set():
+    """`fuse_column_blocks` (no GPU): projections packed side by side share x, so their adapters' A matrices
+    stack along the rank axis and B becomes block-structured; B_fused @ A_fused restricted to a member's rows
+    equals that member's own sum of scaled B_i @ A_i."""
+    import torch
+    from kiln_amd.lora import LoraProjectionWeights, fuse_column_blocks, stack_adapters
+    torch.manual_seed(1)
+    k, widths = 64, (48, 16, 32)
+    mk = lambda n, r: LoraProjectionWeights(torch.randn(r, k).to(torch.bfloat16), torch.randn(n, r).to(torch.bfloat16))
+    q = stack_adapters([mk(48, 4), mk(48, 8)], [0.5, 2.0])
+    v = mk(32, 4)
+    fused = fuse_column_blocks([q, None, v], widths, lora_scale=3.0)
+    assert fused.ranks == (4, 8, 4) and fused.scales == (0.5, 2.0, 3.0)
+    assert tuple(fused.a_cat.shape) == (16, k) and tuple(fused.b_cat.shape) == (96, 16)
+    scale_cols = torch.tensor([0.5] * 4 + [2.0] * 8 + [3.0] * 4)
+    delta = (fused.b_cat.float() * scale_cols) @ fused.a_cat.float()
+    want_q = (q.b_cat.float() * torch.tensor([0.5] * 4 + [2.0] * 8)) @ q.a_cat.float()
+    assert torch.allclose(delta[:48], want_q, rtol=1e-5, atol=1e-5) and torch.count_nonzero(delta[48:64]) == 0
+    assert torch.allclose(delta[64:], 3.0 * (v.b.float() @ v.a.float()), rtol=1e-5, atol=1e-5)
+    assert fuse_column_blocks([None, None], (8, 8)) is None
+    with pytest.raises(marlin_proj.MarlinProjError):
+        fuse_column_blocks([v, None], (48, 16))
