@@ -80,6 +80,7 @@ TUNING_EXPORTS = (
     "kiln_w4a16_debug_prefill_bm", "kiln_w4a16_debug_prefill_nb_full", "kiln_w4a16_debug_decode_direct_max_m",
     "kiln_w4a16_debug_decode_group_major", "kiln_w4a16_debug_decode_runs_per_launch", "kiln_w4a16_debug_tune",
     "kiln_w4a16_debug_mid", "kiln_w4a16_debug_gmp", "kiln_w4a16_debug_flagged", "kiln_w4a16_debug_lora_fold",
+    "kiln_w4a16_debug_rowsum_fold",
 )
 
 _libs: dict[bool, ctypes.CDLL] = {}
@@ -121,6 +122,7 @@ def use_shipped() -> None:
         L.kiln_w4a16_debug_gmp(0, 0, 0)
         L.kiln_w4a16_debug_flagged(-1)
         L.kiln_w4a16_debug_lora_fold(-1)
+        L.kiln_w4a16_debug_rowsum_fold(-1)
     _active_tuning = False
 
 
@@ -161,6 +163,8 @@ def _load(tuning: bool) -> ctypes.CDLL:
     L.kiln_w4a16_debug_decode_plan.argtypes = [i, i, i, i, c.POINTER(c.c_int)]
     L.kiln_w4a16_debug_gemm_plan.restype = i
     L.kiln_w4a16_debug_gemm_plan.argtypes = [i, i, i, i, c.POINTER(c.c_int)]
+    L.kiln_w4a16_debug_prefill_rowsum_producers.restype = i
+    L.kiln_w4a16_debug_prefill_rowsum_producers.argtypes = [i, i, i, i]
     L.kiln_w4a16_gemm_lora.restype = i
     L.kiln_w4a16_gemm_lora.argtypes = [vp, vp, vp, vp, i, i, i, vp, i, i, vp, vp, vp, i, i,
                                        c.POINTER(c.c_int), c.POINTER(c.c_float)]

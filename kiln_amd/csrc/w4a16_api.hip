@@ -75,6 +75,7 @@ struct Tuning {
     int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
     int flagged = -1;                 // 0 = K slices always meet through counters, -1 = automatic
     int lora_fold = -1;               // 0 = the LoRA projection always runs as a launch of its own, -1 = automatic
+    int rowsum_fold = -1;             // 0 = the matrix-core kernel's row sums always come from a launch in front, -1 = automatic
 };
 #ifdef KILN_W4A16_TUNING_HOOKS
 Tuning g_tune;
@@ -728,6 +729,8 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             pa.ranks = lora->ranks;
             pa.scales = lora->scales;
             if (g_tune.lora_fold != 0) pa.lora_words = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
+        } else if (g_tune.rowsum_fold != 0) {
+            pa.lora_words = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
         }
         pa.swiglu = swiglu;
         pa.cus = cus;
@@ -1035,6 +1038,16 @@ int kiln_w4a16_debug_gemm_plan(int m, int n, int k, int cus, int *out) {
     return 0;
 }
 
+// blocks of a plain GEMM of these sizes that form the matrix-core kernel's row sums inside its launch
+// (0: they come from a launch in front, from the blocks themselves, or another kernel runs)
+int kiln_w4a16_debug_prefill_rowsum_producers(int m, int n, int k, int cus) {
+    if (m < 1 || cus < 1 || !shape_ok(n, k, 128)) return -1;
+    GemmPlan gp;
+    plan_gemm(m, n, k, cus, -1, -1, false, &gp);
+    if (!gp.prefill || g_tune.rowsum_fold == 0) return 0;
+    return prefill_rowsum_producers(m, n, k, gp.pf, cus);
+}
+
 #ifdef KILN_W4A16_TUNING_HOOKS
 // Only in the tuning build of the library (never in the shipped one): process-wide overrides of
 // the automatic plan for the test suite and profiling scripts (0 / -1 = automatic).  Plain
@@ -1059,6 +1072,7 @@ void kiln_w4a16_debug_gmp(int tiles, int waves, int kslices) {
 }
 void kiln_w4a16_debug_flagged(int mode) { g_tune.flagged = mode; tuning_changed(); }
 void kiln_w4a16_debug_lora_fold(int mode) { g_tune.lora_fold = mode; }
+void kiln_w4a16_debug_rowsum_fold(int mode) { g_tune.rowsum_fold = mode; }
 void kiln_w4a16_debug_mid(int mode, int pairs, int kslices) {
     g_tune.mid = mode;
     g_tune.mid_pairs = pairs;

@@ -32,6 +32,7 @@
 #include "launch.h"
 #include "lora_tail.h"
 #include "lora_project.h"
+#include "async_loads.h"
 
 namespace kiln {
 
@@ -144,6 +145,10 @@ __device__ __forceinline__ float dpp_move(float v) {
 // workspace that is all zero between launches (the region lora_tail.h describes: the tile words
 // from word kPrefillFoldTileWord of its first replica on); every block counts itself after its
 // look, on the replicated counts, and the last one zeroes words and counts.
+// A launch without adapters uses the same words for the row sums alone (a_cat == nullptr): its
+// producers run rowsum_producer_block.  A block asks for its words a few groups before its main
+// loop ends, with a load that lands in LDS by itself (prefill_fold_peek), and waits for them behind
+// the loop only if that look came too early.
 struct PrefillFold {
     const uint16_t *a_cat;   // bf16 [r_total, K]
     uint16_t *t;             // bf16 [M, RP], behind it the f32 tiles in which K slices meet
@@ -154,11 +159,73 @@ struct PrefillFold {
     int producers;           // row_tiles * kz rounded up to a multiple of 8 (the product's blocks keep their dies)
     int row_tiles, kz, steps_per_slice;
     int consumers;           // blocks of the product (grid padding included)
+    int sum_tiles;           // a_cat == nullptr (no adapters): the producers form the row sums only, this many
+                             // 16-row tiles each
     LoraScales ls;
 };
 constexpr int kPrefillFoldTileWord = 32;
 constexpr int kPrefillFoldMaxTiles = kLoraFoldReplicaWords - kPrefillFoldTileWord;
 constexpr int kPrefillFoldSpinLimit = 1 << 20;
+// where a wavefront's early look at its words lands: the last KiB of the LDS every instance that takes part has
+// (the projection's blocks need kProjectLdsBytes16), behind the A ring and the row sums a block may keep there
+constexpr int kProjectLdsBytes16 = (16 + kProjectMaxRank) * kProjectRowBytes + kProjectMaxRank * (int)sizeof(float);
+constexpr int kFoldPeekOffset = kProjectLdsBytes16 - 1024;
+
+// The row sums of a launch without adapters, as the work of one of its first blocks: the extension
+// operand of 16-row tiles [t0, t1) -- a contiguous piece of A, streamed with 24 loads per thread in
+// flight; 16 lanes per (row, group), the order of additions of w4a16_prefill_rowsum_kernel, whose
+// launch this saves -- written through to memory, then the tiles' words.
+__device__ __forceinline__ void rowsum_producer_block(const uint16_t *__restrict__ A, u32x4 *__restrict__ aext, int M,
+                                                      int K, int t0, int t1, unsigned *done) {
+    constexpr int U = 24;
+    const int G = K / kGroupK;
+    const int r0 = t0 * 16, r1 = min(t1 * 16, M);
+    const int items = (r1 - r0) * G;  // item L: the 256 bytes from byte 256 L of the piece on
+    const int tid = threadIdx.x, sub = tid & 15, slot = tid >> 4;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(A + (size_t)r0 * K) + sub;
+    for (int base = 0; base < items; base += 16 * U) {
+        u32x4 v[U];
+        float sum[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u)  // items past the end re-read the last one
+            v[u] = async_load_b128(src + (size_t)min(base + u * 16 + slot, items - 1) * 16);
+        unrolled<0, U>([&](auto uc) {
+            constexpr int u = decltype(uc)::value;
+            // loads complete in issue order: load u has landed when at most the U - 1 - u later ones are pending
+            __builtin_amdgcn_s_waitcnt(vmcnt_imm(U - 1 - u));
+            pin(v[u]);
+            sum[u] = sum_bf16x8(v[u]);
+#pragma unroll
+            for (int off = 8; off >= 1; off >>= 1) sum[u] += __shfl_xor(sum[u], off, 16);
+        });
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int L = base + u * 16 + slot;
+            if (sub == 0 && L < items) {
+                const int row = L / G, g = L - row * G;
+                store_b128_through(aext + (size_t)g * M + r0 + row, extension_operand(sum[u]));
+            }
+        }
+    }
+    // every wavefront's stores acknowledged, then the words
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0)
+    __syncthreads();
+    for (int t = t0 + tid; t < t1; t += 256) __hip_atomic_store(done + t, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// A look at the words of rows [m0, m0 + rows) that nobody waits for: one device-scope load per lane
+// straight into LDS (256 bytes per wavefront at lds_addr), asked for a few groups before the main
+// loop ends so that the round trip runs under its products; prefill_fold_seen() reads the answer.
+// Every lane must see a raised word: lanes beyond the last tile look at the last one.
+__device__ __forceinline__ void prefill_fold_peek(const PrefillFold &pf, int m0, int rows, int lane, unsigned lds_addr) {
+    const int t0 = m0 >> 4, nt = min((rows + 15) >> 4, pf.row_tiles - t0);
+    const unsigned *p = pf.words + kPrefillFoldTileWord + t0 + min(lane, nt - 1);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off sc1" : : "v"(p), "s"(lds_addr) : "memory", "m0");
+}
+__device__ __forceinline__ bool prefill_fold_seen(const unsigned char *lds_slot, int lane) {
+    const unsigned f = *reinterpret_cast<const volatile unsigned *>(lds_slot + lane * 4);
+    return __builtin_amdgcn_ballot_w64(f == 0u) == 0;
+}
 
 // rows [m0, m0 + rows) of T and of the extension operand are in memory
 __device__ __forceinline__ void prefill_fold_wait(const PrefillFold &pf, int m0, int rows, int lane) {
@@ -205,6 +272,13 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     if constexpr (FOLD) {
         if ((int)blockIdx.x < pf.producers) {
             const int unit = blockIdx.x;
+            if (pf.a_cat == nullptr) {
+                const int t0 = unit * pf.sum_tiles;
+                if (t0 < pf.row_tiles)
+                    rowsum_producer_block(A, pf.aext, M, K, t0, min(t0 + pf.sum_tiles, pf.row_tiles),
+                                          pf.words + kPrefillFoldTileWord);
+                return;
+            }
             if (unit < pf.row_tiles * pf.kz)
                 lora_project_block<16>(lds, A, pf.a_cat, pf.t, M, K, r_total, RP, pf.steps_per_slice, pf.ls, pf.partial,
                                        pf.counters, pf.aext, unit % pf.row_tiles, unit / pf.row_tiles, pf.kz,
@@ -364,6 +438,7 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     // RS: c[group][row] = -136 * (row sum of the group), f32, behind the ring
     [[maybe_unused]] float gsum[RS ? RPW / 16 : 1] = {};
     [[maybe_unused]] float *csum = reinterpret_cast<float *>(lds + kAStages * kAStageBytes);
+    [[maybe_unused]] const int g_peek = max(g_begin, g_end - 3);
     for (int g = g_begin; g < g_end; ++g) {
         const bool more = g + 1 < g_end;
 #pragma unroll
@@ -377,6 +452,11 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
                     bw_next[ni][1] = async_load_b128(b_src[ni][1] + (size_t)(g + 1) * 64);
                     sc_raw_next[ni] = async_load_u16(s_src[ni] + (size_t)((g + 1) & gs_mask) * kTileN);
                 }
+            }
+            if constexpr (FOLD) {
+                // (one more load in flight only makes the counted waits below stricter)
+                if (q == 0 && g == g_peek)
+                    prefill_fold_peek(pf, m0, min(BM, M - m0), lane, lds_base + kFoldPeekOffset + wave * 256);
             }
             const unsigned char *slot = lds + (st & 3) * kAStageBytes;
             // Two k16 steps per stage (step u = 2q + sp uses word q of load sp).
@@ -494,7 +574,8 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     if constexpr (RS) __syncthreads();  // every wavefront's row sums are in LDS
     if constexpr (FOLD) {
         // the rows of this block in the extension operand and in T: written during this launch
-        prefill_fold_wait(pf, m0, min(BM, M - m0), lane);
+        // (the last group's waits have drained every load, the early look included)
+        if (!prefill_fold_seen(lds + kFoldPeekOffset + wave * 256, lane)) prefill_fold_wait(pf, m0, min(BM, M - m0), lane);
         if (wave == 0) prefill_fold_done(pf, consumer, lane);
     }
     // --- remove the 136 * sum(a) * scale surplus: extension contraction ------
@@ -869,7 +950,6 @@ namespace {
 constexpr int kMaxRowSumBytes = 24 * 1024;
 static int row_sum_bytes(int groups) { return groups * 64 * (int)sizeof(float); }
 
-constexpr int kProjectLdsBytes16 = (16 + kProjectMaxRank) * kProjectRowBytes + kProjectMaxRank * (int)sizeof(float);
 
 template <int NWN, int WM, int MI, bool SWIGLU, bool RS, bool FOLD = false>
 hipError_t launch_shape_as(const PrefillArgs &a, int grid, int m_blocks, int RP, int KS, int GSb, int max_groups,
@@ -988,22 +1068,54 @@ hipError_t launch_lora_project(const PrefillArgs &a, bool few_rows, hipStream_t 
     return hipGetLastError();
 }
 
+// 64-row blocks form the row sums themselves when they fit next to the A ring and the launch is
+// bound by latency rather than by work (measured: -2...-10 % up to about 28 GFLOP or on narrow
+// outputs, +6...+8 % beyond, where the extra VALU and LDS work in the main loop costs more
+// than the saved pre-pass launch)
+static bool blocks_sum_their_rows(int M, int N, int K, const PrefillPlan &p) {
+    const int G = K / kGroupK, ks = p.ks < 1 ? 1 : p.ks;
+    // most groups of K any one block covers: all of them for a whole tile
+    const int max_groups = p.nb_full > 0 ? G : (G + ks - 1) / ks;
+    const double flops = 2.0 * M * (double)N * K;
+    return p.bm == 64 && row_sum_bytes(max_groups) <= kMaxRowSumBytes && (flops <= 28e9 || N <= 4096);
+}
+
+// Without adapters a few of the product's own first blocks form the row sums (rowsum_producer_block)
+// where the launch is a single round of blocks that leaves block slots free: producers in those
+// slots cost the product nothing and save the launch in front (down projection at 2048 rows
+// 116 -> 112 us, 2560 -> 8192 at 777 rows 61 -> 59.5).  They must be done before the first block's main
+// loop is: at least one per 64 rows (its piece of A then streams in about half that time, whatever
+// K), as many as there are free slots up to one per 16-row tile.  In a launch of several rounds the
+// producers' slots are taken from the product: measured 2 to 5 us slower than the launch in front
+// (gate+up at 2048 and 4096 rows), so those keep it.  0: the row sums come from elsewhere.
+int prefill_rowsum_producers(int M, int N, int K, const PrefillPlan &p, int cus) {
+    if (blocks_sum_their_rows(M, N, K, p) || p.bn != 256 || (p.bm != 64 && p.bm != 128) ||
+        (M + 15) / 16 > kPrefillFoldMaxTiles || p.nb_full < 0 || p.nb_full > N / p.bn)
+        return 0;
+    const int grid = prefill_grid(M, N, p), slots = cus * (p.bm == 128 ? 2 : 3);
+    const int want = ((M + 63) / 64 + 7) / 8 * 8, tiles8 = ((M + 15) / 16 + 7) / 8 * 8;
+    const int free_slots = (slots - grid) / 8 * 8;
+    if (free_slots < want) return 0;
+    const int producers = free_slots < tiles8 ? free_slots : tiles8;
+    return producers < 128 ? producers : 128;
+}
+
 hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     const int G = a.K / kGroupK;
     if (a.bm != 64 && a.bm != 128 && a.bm != 256) return hipErrorInvalidValue;
     const int KS_ = a.KS < 1 ? 1 : a.KS;
-    // most groups of K any one block covers: all of them for a whole tile
+    PrefillPlan shape;
+    shape.bn = a.bn;
+    shape.bm = a.bm;
+    shape.ks = KS_;
+    shape.nb_full = a.nb_full;
     const int max_groups = a.nb_full > 0 ? G : (G + KS_ - 1) / KS_;
-    // 64-row blocks form the row sums themselves when they fit next to the A ring and the launch is
-    // bound by latency rather than by work (measured: -2...-10 % up to about 28 GFLOP or on narrow
-    // outputs, +6...+8 % beyond, where the extra VALU and LDS work in the main loop costs more
-    // than the saved pre-pass launch)
-    const double flops = 2.0 * a.M * (double)a.N * a.K;
-    const bool rs = a.bm == 64 && row_sum_bytes(max_groups) <= kMaxRowSumBytes && (flops <= 28e9 || a.N <= 4096);
+    const bool rs = blocks_sum_their_rows(a.M, a.N, a.K, shape);
     hipError_t err = hipSuccess;
     // with adapters the projection's launch forms the row sums on its way over x
     const bool sums_with_projection = !rs && a.r_total > 0;
-    if (!rs && !sums_with_projection) {
+    const int sum_producers = a.r_total == 0 && a.lora_words ? prefill_rowsum_producers(a.M, a.N, a.K, shape, a.cus) : 0;
+    if (!rs && !sums_with_projection && sum_producers == 0) {
         const int items = a.M * G;
         w4a16_prefill_rowsum_kernel<<<(items + 15) / 16, 256, 0, stream>>>((const uint16_t *)a.A, (u32x4 *)a.aext,
                                                                           a.M, a.K);
@@ -1050,16 +1162,19 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
             if (slices != 1) return hipErrorInvalidValue;
         }
     }
+    if (sum_producers > 0) {
+        fold = true;
+        pf.aext = (u32x4 *)a.aext;
+        pf.words = a.lora_words;
+        pf.row_tiles = (a.M + 15) / 16;
+        pf.producers = sum_producers;
+        pf.sum_tiles = (pf.row_tiles + sum_producers - 1) / sum_producers;
+    }
     if (a.bn != 128 && a.bn != 256) return hipErrorInvalidValue;
     const int m_blocks = (a.M + a.bm - 1) / a.bm;
     const int KS = a.KS < 1 ? 1 : a.KS;
     const int GSb = (G + KS - 1) / KS;
     if (KS > 1 && (!a.partial || !a.counters || (KS - 1) * GSb >= G)) return hipErrorInvalidValue;
-    PrefillPlan shape;
-    shape.bn = a.bn;
-    shape.bm = a.bm;
-    shape.ks = KS;
-    shape.nb_full = a.nb_full;
     if (a.nb_full < 0 || a.nb_full > a.N / a.bn) return hipErrorInvalidValue;
     const int grid = prefill_grid(a.M, a.N, shape);
     if (fold) {
