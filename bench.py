@@ -90,8 +90,16 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
     for name, (k, n) in shapes.items():
         us = time_shape(2048, k, n, 72)
         tf = 2 * 2048 * k * n / us / 1e6
+        # what a call launches: the product, and where its row sums (operand of the offset removal) come from
+        from kiln_amd import _lib
+        cus_ = torch.cuda.get_device_properties(dev).multi_processor_count
+        src_ = _lib.load().kiln_w4a16_debug_prefill_rowsum_producers(2048, n, k, cus_)
         extra[f"cfg2_m2048_{name}"] = {"us": round(us, 2), "TFLOPs": round(tf, 1),
-                                       "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4)}
+                                       "mfma_frac": round(tf / MFMA_BF16_PEAK_TFLOPS, 4),
+                                       "launches_per_call": 2 if src_ == 0 else 1,
+                                       "row_sums": ("a launch in front (its time is included)" if src_ == 0 else
+                                                    f"{src_} blocks of the product's own launch" if src_ > 0 else
+                                                    "inside the product's blocks")}
     # cfg 4: prefill with two stacked LoRA adapters fused into the epilogue
     ranks, lscales = (16, 32), (0.5, 1.0)
     la = (torch.randn(sum(ranks), 2560, device=dev) * 0.02).to(torch.bfloat16)
@@ -286,7 +294,9 @@ def main() -> int:
     ap.add_argument("--profile", choices=["decode", "decode_m1", "mid", "prefill", "lora", "pack"], default=None,
                     help="for rocprofv3: launch K eager steps of the chosen regime (no graph, no CPU "
                          "baseline, no extra legs) plus one 64 MiB device copy that calibrates the "
-                         "memory-traffic counters, print no JSON; decode_m1: gate+up, down and the "
+                         "memory-traffic counters, print no JSON; prefill: the two cfg 2 GEMMs at M=2048, "
+                         "K calls each in a captured graph replayed twice, as the legs under `extra` run "
+                         "them; decode_m1: gate+up, down and the "
                          "2560x2560 GEMV at M=1; mid: the four projection shapes of the sweep at M=64; "
                          "lora: the decode step and the M=512 gate+up GEMM, each with two stacked "
                          "adapters (ranks 16 and 32)")
@@ -391,12 +401,33 @@ def main() -> int:
                 marlin_gemm.marlin_w4a16_gemm_lora(x512, b, s, GROUP, ad["gate_up"][0], ad["gate_up"][1], ranks,
                                                    lscales, out=o512)
         else:
+            # as the cfg 2 legs under `extra` run them: one captured graph per shape, the calls back to back,
+            # replayed once untimed and once between events (the tracer spaces the nodes out, so the figure
+            # printed here is an upper bound; the trace's durations are the kernels' own)
             xp = {name: torch.randn(2048, kn[0], device=dev).to(torch.bfloat16) for name, kn in shapes.items()}
             op = {name: torch.empty(2048, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in shapes.items()}
-            for i in range(args.steps):
-                for name in shapes:
+            side = torch.cuda.Stream()
+            for name in shapes:
+                def call(i, name=name):
                     b, s = layers[i % LAYERS][name]
                     marlin_gemm.marlin_w4a16_gemm(xp[name], b, s, GROUP, out=op[name])
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.stream(side):
+                    for i in range(LAYERS):
+                        call(i)
+                    side.synchronize()
+                    with torch.cuda.graph(g, stream=side):
+                        for i in range(args.steps):
+                            call(i)
+                    g.replay()
+                    side.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record(side)
+                    g.replay()
+                    e1.record(side)
+                    side.synchronize()
+                print(f"bench.py --profile prefill: {name} M=2048, {args.steps} calls per replay, "
+                      f"{e0.elapsed_time(e1) * 1e3 / args.steps:.2f} us per call between events", file=sys.stderr)
         torch.cuda.synchronize()
         return 0
 

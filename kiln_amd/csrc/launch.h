@@ -194,7 +194,7 @@ struct PrefillPlan {
 PrefillPlan plan_prefill(int m, int n, int k, int cus, int force_bn = 0, int force_bm = 0);
 int prefill_grid(int m, int n, const PrefillPlan &p);
 size_t prefill_partial_bytes(int m, int n, const PrefillPlan &p);
-int prefill_rowsum_producers(int m, int n, int k, const PrefillPlan &p, int cus);  // blocks of a plain launch that form the row sums inside it (0: none)
+int prefill_rowsum_producers(int m, int n, int k, const PrefillPlan &p, int cus);  // blocks of a plain launch that form the row sums inside it (0: a launch in front does, -2: every block its own)
 hipError_t launch_prefill(const PrefillArgs &args, hipStream_t stream);
 // lora_t = bf16 [*slices][M][r_total rounded up to 16] = per-adapter scale * (A * lora_a^T) in K slices,
 // padding columns zero.  few_rows: the small-M kernels will multiply it, in up to

@@ -1038,14 +1038,16 @@ int kiln_w4a16_debug_gemm_plan(int m, int n, int k, int cus, int *out) {
     return 0;
 }
 
-// blocks of a plain GEMM of these sizes that form the matrix-core kernel's row sums inside its launch
-// (0: they come from a launch in front, from the blocks themselves, or another kernel runs)
+// Where the matrix-core kernel's row sums come from on a plain GEMM of these sizes: > 0 = that many blocks
+// of its own launch, 0 = a launch in front, -2 = every block sums its own rows, -3 = another kernel runs;
+// -1 = bad sizes
 int kiln_w4a16_debug_prefill_rowsum_producers(int m, int n, int k, int cus) {
     if (m < 1 || cus < 1 || !shape_ok(n, k, 128)) return -1;
     GemmPlan gp;
     plan_gemm(m, n, k, cus, -1, -1, false, &gp);
-    if (!gp.prefill || g_tune.rowsum_fold == 0) return 0;
-    return prefill_rowsum_producers(m, n, k, gp.pf, cus);
+    if (!gp.prefill) return -3;
+    const int inside = prefill_rowsum_producers(m, n, k, gp.pf, cus);
+    return inside > 0 && g_tune.rowsum_fold == 0 ? 0 : inside;
 }
 
 #ifdef KILN_W4A16_TUNING_HOOKS

@@ -1087,9 +1087,11 @@ static bool blocks_sum_their_rows(int M, int N, int K, const PrefillPlan &p) {
 // loop is: at least one per 64 rows (its piece of A then streams in about half that time, whatever
 // K), as many as there are free slots up to one per 16-row tile.  In a launch of several rounds the
 // producers' slots are taken from the product: measured 2 to 5 us slower than the launch in front
-// (gate+up at 2048 and 4096 rows), so those keep it.  0: the row sums come from elsewhere.
+// (gate+up at 2048 and 4096 rows), so those keep it.  0: from the launch in front; -2: the blocks sum
+// their rows themselves.
 int prefill_rowsum_producers(int M, int N, int K, const PrefillPlan &p, int cus) {
-    if (blocks_sum_their_rows(M, N, K, p) || p.bn != 256 || (p.bm != 64 && p.bm != 128) ||
+    if (blocks_sum_their_rows(M, N, K, p)) return -2;
+    if ( p.bn != 256 || (p.bm != 64 && p.bm != 128) ||
         (M + 15) / 16 > kPrefillFoldMaxTiles || p.nb_full < 0 || p.nb_full > N / p.bn)
         return 0;
     const int grid = prefill_grid(M, N, p), slots = cus * (p.bm == 128 ? 2 : 3);
@@ -1114,7 +1116,8 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
     hipError_t err = hipSuccess;
     // with adapters the projection's launch forms the row sums on its way over x
     const bool sums_with_projection = !rs && a.r_total > 0;
-    const int sum_producers = a.r_total == 0 && a.lora_words ? prefill_rowsum_producers(a.M, a.N, a.K, shape, a.cus) : 0;
+    const int inside = a.r_total == 0 && a.lora_words ? prefill_rowsum_producers(a.M, a.N, a.K, shape, a.cus) : 0;
+    const int sum_producers = inside > 0 ? inside : 0;
     if (!rs && !sums_with_projection && sum_producers == 0) {
         const int items = a.M * G;
         w4a16_prefill_rowsum_kernel<<<(items + 15) / 16, 256, 0, stream>>>((const uint16_t *)a.A, (u32x4 *)a.aext,

@@ -23,6 +23,7 @@ CASES = [
     (2048, 2560, 18432, False),  # several rounds of blocks: the launch in front stays
     (300, 2560, 2560, False),    # the blocks sum their rows themselves
 ]
+IN_FRONT, OWN_ROWS, OTHER_KERNEL = 0, -2, -3
 
 
 def _cus():
@@ -36,9 +37,12 @@ def test_the_plan_query_says_where_the_row_sums_come_from():
         assert (p > 0) == inside, (m, k, n, p)
         if inside:
             assert p % 8 == 0 and 8 <= p <= 128 and p >= (m + 63) // 64
+    assert L.kiln_w4a16_debug_prefill_rowsum_producers(2048, 18432, 2560, _cus()) == IN_FRONT
+    assert L.kiln_w4a16_debug_prefill_rowsum_producers(300, 2560, 2560, _cus()) == OWN_ROWS
+    assert L.kiln_w4a16_debug_prefill_rowsum_producers(16, 2560, 2560, _cus()) == OTHER_KERNEL
     try:
         L.kiln_w4a16_debug_rowsum_fold(0)
-        assert L.kiln_w4a16_debug_prefill_rowsum_producers(2048, 2560, 9216, _cus()) == 0
+        assert L.kiln_w4a16_debug_prefill_rowsum_producers(2048, 2560, 9216, _cus()) == IN_FRONT
     finally:
         L.kiln_w4a16_debug_rowsum_fold(-1)
     assert L.kiln_w4a16_debug_prefill_rowsum_producers(0, 2560, 9216, _cus()) == -1
