@@ -259,7 +259,9 @@ bool flagged_exchange_fits(int ks, int n) {
 }
 
 // Best plan for the private-staging group-major instance (m <= 16).  Cost in microseconds, fitted
-// to sweeps of the model's projection shapes at 1, 4, 8 and 16 rows: a launch costs about 2.8 us
+// to sweeps of the model's projection shapes at 1, 4, 8 and 16 rows and checked against sweeps of
+// every plan on 24 shapes (those, the side-by-side packs, and 18 of other models: 1536 ... 28672 wide),
+// where the plan it picks is 1.4 % slower than the best forced plan on average and 13 % at worst: a launch costs about 2.8 us
 // beside its rounds of blocks; a block streams its T * GS KiB of weights at 0.036 us per KiB and
 // stages its rows of A from L2 (GS KiB per four rows) at 0.0125 us per KiB -- with 16 rows an
 // unsliced down projection stages four times the bytes it streams, which is why it is sliced there
@@ -280,9 +282,12 @@ bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) 
         for (int waves : kWaves) {
             for (int T = 1; T <= 6; ++T) {
                 // 16 wavefronts only where they take one tile and the same number of groups each
-                // (out-projection: 4.9 against 5.3 us with 12); elsewhere they measured slower
-                if (waves == 16 && (T != 1 || GS % 16 != 0)) continue;
+                // (out-projection: 4.9 against 5.3 us with 12), or where 12 cannot form the plan (a
+                // wavefront holds at most 16 chunks: 5120 -> 13824 in blocks of four tiles, one round,
+                // 8.4 us at one row against 10.4 in two rounds of two-tile blocks); elsewhere they
+                // measured 5 to 15 % slower than 12 on the same tiles and slices
                 DecodePlan p;
+                if (waves == 16 && (T != 1 || GS % 16 != 0) && gmp_plan(m, n, k, T, 12, ks, lora, &p)) continue;
                 if (!gmp_plan(m, n, k, T, waves, ks, lora, &p)) continue;
                 const int rounds = ceil_div(ceil_div(NT, T) * ks, cus);
                 // The exchange: through counters 0.4 us per slice + 1.2; with the parts as their own
@@ -295,8 +300,14 @@ bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) 
                 const bool flagged = flagged_exchange_fits(ks, n);
                 const float exchange = ks == 1 ? 0.f : (flagged ? 0.4f + 0.0037f * (ks - 1) * NT : 0.4f * ks + 1.2f) +
                                                            (a_kib_per_group == 1 ? 0.7f : 0.f);
-                const float cost = 2.8f + rounds * (0.036f * T * GS + 0.0125f * a_kib_per_group * GS) +
-                                   0.08f * T * ceil_div(GS, p.waves) + exchange;
+                // Every round after the first costs its blocks' start on top (1 us: 4096 -> 14336 at one row
+                // 9.8 us in two rounds of two-tile blocks, 7.5 in one round of four-tile blocks).  Eight
+                // wavefronts with three or more tiles each measure 3 to 7 % below twelve on the same
+                // tiles (fewer partial tiles to add at the end: gate+up at 16 rows 7.9 -> 7.6 us,
+                // q|k|v side by side 6.5 -> 6.15); with adapters the twelve stay (not measured).
+                float cost = 2.8f + rounds * (0.036f * T * GS + 0.0125f * a_kib_per_group * GS) +
+                             0.08f * T * ceil_div(GS, p.waves) + exchange + 1.0f * (rounds - 1);
+                if (waves == 8 && T >= 3 && !lora) cost *= 0.95f;
                 if (best_cost < 0.f || cost < best_cost - 1e-4f) {
                     best_cost = cost;
                     *best = p;
