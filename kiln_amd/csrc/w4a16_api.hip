@@ -496,7 +496,11 @@ bool mid_flagged(const MidArgs &a) {
 // parallelism for L2 traffic); a launch costs about 4.5 us beside its rounds of blocks, an exchange
 // between K slices through counters 1.5 us at two slices and 1.7 us more per further slice
 // (out-projection at 64 rows: 11.5 us unsliced, 10.4 in two slices, 13.8 in four), the counter-free
-// exchange 1 us less (9.4 in two slices).
+// exchange 1 us less (9.4 in two slices).  Every round of blocks after the first costs its start on top
+// (2 us: without it many rounds of short slices looked cheap -- 5120 -> 13824 at 128 rows 58 us in five
+// slices against 48 in two).  Checked against every forced plan on 20 shapes (those four, the
+// side-by-side packs and 14 of other models) at 40, 64, 96 and 128 rows: the plan picked is 1.6 %
+// slower than the best on average, 25 % at worst (4096 -> 1024, where four slices would beat two).
 MidPlan plan_mid(int m, int n, int k, int cus) {
     MidPlan best;
     const int G = k / kGroupK, runs = ceil_div(m, mid_max_rows_per_run());
@@ -517,7 +521,7 @@ MidPlan plan_mid(int m, int n, int k, int cus) {
             if ((size_t)runs * col_blocks * sizeof(int) > kCounterCapacity) continue;
             const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
             const float exchange = ks == 1 ? 0.f : (mid_flagged(a) ? 1.7f * ks - 2.9f : 1.7f * ks - 1.9f);
-            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange;
+            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange + 2.0f * (rounds - 1);
             if (!best.ok || cost < best.cost) {
                 best.ok = true;
                 best.KS = ks;

@@ -892,10 +892,16 @@ static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm, 
 // Relative cost of a plan in units of one 128-column block's group: whole rounds, then the
 // sliced round, then the exchange of its partial tiles (wider blocks take about 1.3 times as
 // long per group and exchange twice the data).
+// A 128-row block takes 1.5 times as long per group as a 64-row one, exchanges at twice the price per
+// slice, and its launch carries 8 units more (the row sums from a launch in front, a longer prologue and
+// store): fitted to 98 cases -- 14 shapes at 400 ... 4096 rows, each with 64- and 128-row blocks forced --
+// on which the cheaper plan by this cost is the faster one or within 0.8 % of it on average (14 % at worst).
 static float plan_cost(int m, int n, int k, int cus, const PrefillPlan &p) {
     const int G = k / kGroupK, m_blocks = (m + p.bm - 1) / p.bm, n_blocks = n / p.bn;
-    const float per_group = p.bn == 256 ? 1.3f : 1.0f, per_slice = p.bn == 256 ? 1.0f : 0.5f;
-    float cost = (float)((m_blocks * n_blocks) / cus) * G * per_group;
+    const float rows = p.bm == 128 ? 1.5f : 1.0f;
+    const float per_group = (p.bn == 256 ? 1.3f : 1.0f) * rows;
+    const float per_slice = (p.bn == 256 ? (p.bm == 128 ? 2.0f : 1.0f) : 0.5f) * rows;
+    float cost = (float)((m_blocks * n_blocks) / cus) * G * per_group + (p.bm == 128 ? 8.f : 0.f);
     if (n_blocks > p.nb_full) {
         cost += (float)((G + p.ks - 1) / p.ks) * per_group;
         if (p.ks > 1) cost += per_slice * p.ks;
@@ -903,41 +909,51 @@ static float plan_cost(int m, int n, int k, int cus, const PrefillPlan &p) {
     return cost;
 }
 
-// Block shape for a problem, from a sweep of the model's projection shapes over M = 33...4096.
-// Rows: 64-row blocks (four wavefronts side by side, three blocks per compute unit) up to
-// M = 768: small problems are bound by latency and by how evenly the tiles cover the chip,
-// not by the matrix cores, and rows past M are computed and dropped.  Beyond that 128 x 256
-// blocks (four wavefronts side by side, each 128 x 64): the best measured rate when the chip
-// is saturated, because every wavefront's weights are its own and A is shared by all four.
-// Where those tiles would cover between half and all of the compute units and cannot be
-// sliced, 64 x 256 blocks cover the chip better.
-// Columns of the 64-row block: whichever of 128 and 256 has the lower modelled cost.
+// Block shape for a problem.  64-row blocks (four wavefronts side by side, three blocks per compute
+// unit) for small problems, which are bound by latency and by how evenly the tiles cover the chip,
+// not by the matrix cores (rows past M are computed and dropped); 128 x 256 blocks (four wavefronts
+// side by side, each 128 x 64) where the chip is saturated: the best measured rate, because every
+// wavefront's weights are its own and A is shared by all four.  Which of the two, and which width
+// of the 64-row block: the lower modelled cost (plan_cost); up to 384 rows always 64.  (A fixed
+// switch at 768 rows was 5 % slower on average over the same 98 cases and 69 % at worst: narrow
+// outputs want 64 rows at any row count, large products 128 rows from 400 on.)
 // The 256-row shapes stay available through the overrides.
 PrefillPlan plan_prefill(int m, int n, int k, int cus, int force_bn, int force_bm) {
-    int bm = m <= 768 ? 64 : 128;
+    // 128-row tiles for 50...100 % of the compute units: two such blocks fit a unit, and with every tile cut
+    // into as many K slices as fill those slots the chip is busier than with 64-row blocks, provided a slice
+    // stays long (measured on N = 2560: K = 9216 at M = 2048 / 2560 / 3072, three or two slices of 24 or 36
+    // groups, 121 / 148 / 162 us against 124 / 159 / 168; K = 4096 at M = 3072 in two slices of 16 groups
+    // 90 against 84)
     int sliced_units = 0;
-    if (bm == 128) {
+    {
         const int tiles = ((m + 127) / 128) * (n / 256);
         if (2 * tiles > cus && tiles < cus) {
-            // Tiles for 50...100 % of the compute units.  Two 128-row blocks fit a unit: with every tile
-            // cut into as many K slices as fill those slots the chip is busier than with 64-row blocks,
-            // provided a slice stays long (measured on N = 2560: K = 9216 at M = 2048 / 2560 / 3072, three
-            // or two slices of 24 or 36 groups, 121 / 148 / 162 us against 124 / 159 / 168; K = 4096 at
-            // M = 3072 in two slices of 16 groups 90 against 84)
             const int ks = 2 * cus / tiles;
             if (ks >= 2 && k / kGroupK / ks >= 24) sliced_units = 2 * cus;
-            else bm = 64;
         }
     }
-    if (force_bm == 64 || force_bm == 128 || force_bm == 256) bm = force_bm;
-    if (force_bn == 128 || force_bn == 256) return plan_for_shape(m, n, k, cus, force_bn, bm);
-    const PrefillPlan wide = plan_for_shape(m, n, k, cus, 256, bm, bm == 128 ? sliced_units : 0);
-    if (bm == 128) return wide;
-    const PrefillPlan narrow = plan_for_shape(m, n, k, cus, 128, bm);
-    if (bm == 64) return plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, wide) ? narrow : wide;
-    // 256-row blocks: narrow unless its tiles neither fill a round nor can be sliced
-    if (narrow.nb_full == 0 && narrow.ks == 1 && wide.nb_full == 0 && wide.ks >= 2) return wide;
-    return narrow;
+    if (force_bm == 64 || force_bm == 128 || force_bm == 256) {
+        const int bm = force_bm;
+        if (force_bn == 128 || force_bn == 256) return plan_for_shape(m, n, k, cus, force_bn, bm);
+        const PrefillPlan wide = plan_for_shape(m, n, k, cus, 256, bm, bm == 128 ? sliced_units : 0);
+        if (bm == 128) return wide;
+        const PrefillPlan narrow = plan_for_shape(m, n, k, cus, 128, bm);
+        if (bm == 64) return plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, wide) ? narrow : wide;
+        // 256-row blocks: narrow unless its tiles neither fill a round nor can be sliced
+        if (narrow.nb_full == 0 && narrow.ks == 1 && wide.nb_full == 0 && wide.ks >= 2) return wide;
+        return narrow;
+    }
+    // 64-row blocks of either width, and from 385 rows on 128 x 256 blocks: whichever the cost model prices lower
+    PrefillPlan best = plan_for_shape(m, n, k, cus, force_bn == 128 ? 128 : 256, 64);
+    if (force_bn != 128 && force_bn != 256) {
+        const PrefillPlan narrow = plan_for_shape(m, n, k, cus, 128, 64);
+        if (plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, best)) best = narrow;
+    }
+    if (m > 384 && force_bn != 128) {
+        const PrefillPlan tall = plan_for_shape(m, n, k, cus, 256, 128, sliced_units);
+        if (plan_cost(m, n, k, cus, tall) < plan_cost(m, n, k, cus, best)) best = tall;
+    }
+    return best;
 }
 size_t prefill_partial_bytes(int m, int n, const PrefillPlan &p) {
     if (p.ks <= 1) return 0;

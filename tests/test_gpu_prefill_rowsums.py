@@ -17,9 +17,10 @@ pytestmark = pytest.mark.gpu
 # (rows, k, n, expected: producers inside the launch)
 CASES = [
     (2048, 9216, 2560, True),    # cfg 2's down projection: 480 blocks of 128 rows on 512 slots
-    (777, 2560, 8192, True),     # ragged rows, 64-row blocks that do not sum their own rows
-    (1536, 4096, 2560, True),
-    (1000, 2560, 1024, True),    # k/v projection width
+    (777, 2560, 8192, True),     # ragged rows
+    (1536, 9216, 2560, True),
+    (600, 2560, 12288, True),    # 128-row blocks below 768 rows
+    (2500, 4096, 2560, True),    # the most producers a launch takes
     (2048, 2560, 18432, False),  # several rounds of blocks: the launch in front stays
     (300, 2560, 2560, False),    # the blocks sum their rows themselves
 ]
