@@ -471,16 +471,31 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
     gp->pf = p;
 }
 
-// Rows the mid-M kernel takes on the automatic plan: above the two-slab small-M instance's 32
-// (up to 32 rows that instance is ahead on every projection shape: 8.5 / 8.4 / 11.3 / 11.6 us
-// against 9.1 / 10.8 / 14.1 / 14.1) and up to two runs of 64 -- three for outputs of up to 8192
-// columns, where it still leads the matrix-core kernel's 64-row blocks at 192 rows (21.3 against
-// 23.8 us on the in-projection, 12.0 against 21.0 on the out-projection) while the widest
-// projection does not (38.8 against 34.5).  With adapters it starts at 17 rows: the two-slab
-// instance needs the projection from a launch in front, the mid-M kernel computes it in its own
-// first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.2 / 12.8 /
-// 16.5 / 16.3 us against 14.4 / 13.3 / 19.2 / 17.0).
-constexpr int kMidMinM = 33, kMidMinMLora = 17, kMidMaxM = 128, kMidMaxMNarrow = 192, kMidNarrowN = 8192;
+// Rows the mid-M kernel takes on the automatic plan, from sweeps of the three kernels forced on 13 shapes
+// (the model's, the side-by-side packs, seven of other models) at 20 ... 320 rows.
+// From: 33 rows -- up to 32 the two-slab small-M instance is ahead wherever K = 2560 (gate+up 11.4 against
+// 14.9 us at 32 rows, in-projection 8.2 against 9.1) -- but 24 rows where K >= 4096, whose longer columns the
+// mid-M kernel's K slices and wider products serve better (4096 -> 14336 at 32 rows 17.4 against 21.3 us,
+// 8192 -> 8192 21.8 against 26.3, down projection 11.6 against 12.5; level at 24).  With adapters 17: the
+// two-slab instance needs the projection from a launch in front, the mid-M kernel computes it in its own
+// first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.2 / 12.8 / 16.5 / 16.3 us
+// against 14.4 / 13.3 / 19.2 / 17.0).
+// To: 128 rows (two runs of 64); small weights keep it ahead of the matrix-core kernel's 64-row blocks for
+// longer -- K * N up to 32 M: 192 rows, 256 where K <= 4096 (in-projection at 256 rows 25.2 against 26.5 us,
+// 2560 -> 12288 31.8 against 35.0, down projection at 192 rows 24.5 against 29.1 but 34.5 against 31.3 at 256);
+// up to 12 M: 320 rows (out-projection at 320 rows 16.1 against 23.1, 2560 -> 1024 8.7 against 16.2) -- while
+// on large ones it falls behind from 160 rows on (14336 -> 4096: 55 against 47 us; gate+up 42.5 against 35.2).
+constexpr int kMidMinM = 33, kMidMinMLongK = 24, kMidMinMLora = 17, kMidMaxM = 128, kMidMaxMSmallest = 320;
+int mid_min_rows(int n, int k, bool lora) {
+    // (beyond 68 M weights the two-slab instance leads again: 5120 -> 13824 at 32 rows 23.3 against 25.9 us)
+    return lora ? kMidMinMLora : (k >= 4096 && (long long)k * n <= (68ll << 20) ? kMidMinMLongK : kMidMinM);
+}
+int mid_max_rows(int n, int k) {
+    const long long kn = (long long)k * n;
+    if (kn <= 12ll << 20) return kMidMaxMSmallest;
+    if (kn <= 32ll << 20) return k <= 4096 ? 256 : 192;
+    return kMidMaxM;
+}
 
 // Do the K slices of this mid-M launch meet in the zeroed region, the parts being their own arrival flags?
 bool mid_flagged(const MidArgs &a) {
@@ -552,9 +567,11 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
     *gp = GemmPlan{};
     // 33...128 rows: the mid-M kernel, one pass over the weights per 64 rows (with adapters whose
     // stacked rank is a multiple of 8: the low-rank term is added from a projection launched in front)
+    // (a call pinned to a block shape of the matrix-core kernel goes there)
+    const bool prefill_pinned = g_tune.prefill_bm != 0 || g_tune.prefill_bn != 0 || g_tune.prefill_ks != 0 || g_tune.prefill_nb_full >= 0;
     if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
         (g_tune.mid == 1 ||
-         (g_tune.prefill_min_m == 0 && m >= (lora ? kMidMinMLora : kMidMinM) && m <= (n <= kMidNarrowN ? kMidMaxMNarrow : kMidMaxM)))) {
+         (!prefill_pinned && g_tune.prefill_min_m == 0 && m >= mid_min_rows(n, k, lora != 0) && m <= mid_max_rows(n, k)))) {
         // with adapters the projection runs in the launch's first blocks: plan for the chip less those
         const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
         const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus);
@@ -684,7 +701,7 @@ struct LoraSpec {
 };
 
 // Bytes a call of m rows needs, made monotone in m: the largest need of any m' <= m.  The plan
-// (and with it the need) changes with m' only through the small-M runs (m' <= 128 here; beyond
+// (and with it the need) changes with m' only through the small-M and mid-M runs (m' <= 320 here; beyond
 // that only overrides keep a call on that path) and through the matrix-core kernel's row blocks
 // of 64 or 128 rows, so those m' are the ones evaluated.
 size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thread_n) {
@@ -697,7 +714,7 @@ size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thre
             if (need > most) most = need;
         }
     };
-    const int small = g_tune.prefill_min_m > kMidMaxMNarrow ? g_tune.prefill_min_m : kMidMaxMNarrow;
+    const int small = g_tune.prefill_min_m > kMidMaxMSmallest ? g_tune.prefill_min_m : kMidMaxMSmallest;
     for (int mm = 1; mm <= m && mm <= small; ++mm) consider(mm);
     for (int mm = 64; mm < m; mm += 64) consider(mm);
     consider(m);
