@@ -36,11 +36,11 @@ LAYERS = 16
 TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median replay is reported
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
-# copy (x1.9989 and x1.0): 12278.6 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
+# copy (x1.9989 and x1.0): 12307.1 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25722600, "kernel": "w4a16_decode_gmp_kernel<5, 2, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25780788, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 
@@ -295,7 +295,7 @@ def main() -> int:
                     help="for rocprofv3: launch K eager steps of the chosen regime (no graph, no CPU "
                          "baseline, no extra legs) plus one 64 MiB device copy that calibrates the "
                          "memory-traffic counters, print no JSON; prefill: the two cfg 2 GEMMs at M=2048, "
-                         "K calls each in a captured graph replayed twice, as the legs under `extra` run "
+                         "K calls each in a captured graph replayed six times, as the legs under `extra` run "
                          "them; decode_m1: gate+up, down and the "
                          "2560x2560 GEMV at M=1; mid: the four projection shapes of the sweep at M=64; "
                          "lora: the decode step and the M=512 gate+up GEMM, each with two stacked "
@@ -402,8 +402,9 @@ def main() -> int:
                                                    lscales, out=o512)
         else:
             # as the cfg 2 legs under `extra` run them: one captured graph per shape, the calls back to back,
-            # replayed once untimed and once between events (the tracer spaces the nodes out, so the figure
-            # printed here is an upper bound; the trace's durations are the kernels' own)
+            # replayed five times untimed (the part needs tens of milliseconds of this load to settle: the
+            # first replays read up to 10 % slower) and once between events (the tracer spaces the nodes out,
+            # so the figure printed here is an upper bound; the trace's durations are the kernels' own)
             xp = {name: torch.randn(2048, kn[0], device=dev).to(torch.bfloat16) for name, kn in shapes.items()}
             op = {name: torch.empty(2048, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in shapes.items()}
             side = torch.cuda.Stream()
@@ -419,14 +420,15 @@ def main() -> int:
                     with torch.cuda.graph(g, stream=side):
                         for i in range(args.steps):
                             call(i)
-                    g.replay()
+                    for _ in range(5):
+                        g.replay()
                     side.synchronize()
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     e0.record(side)
                     g.replay()
                     e1.record(side)
                     side.synchronize()
-                print(f"bench.py --profile prefill: {name} M=2048, {args.steps} calls per replay, "
+                print(f"bench.py --profile prefill: {name} M=2048, {args.steps} calls per replay, sixth replay "
                       f"{e0.elapsed_time(e1) * 1e3 / args.steps:.2f} us per call between events", file=sys.stderr)
         torch.cuda.synchronize()
         return 0
