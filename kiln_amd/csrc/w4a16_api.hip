@@ -393,7 +393,8 @@ SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n,
     return c;
 }
 
-// Does a GEMM of m rows take the matrix-core kernel?  Below the change-over the rows go through
+// Does a GEMM of m rows that the mid-M kernel does not take (plan overrides, adapters of a stacked rank
+// that is not a multiple of 8, shapes without a mid-M plan) take the matrix-core kernel?  Below the change-over the rows go through
 // the small-M kernels in runs, every launch streaming the weights again.  Where a plan for the
 // two-slab small-M instance exists, up to 80 rows go there (runs of 32 rows, up to four per
 // launch); measured against the matrix-core kernel's 64-row blocks (16-24 us at any M <= 64) it is

@@ -14,9 +14,11 @@
 //     K: the down projection runs unsliced, without the exchange through the workspace;
 //   * the weight requests are the first memory instructions of the kernel, ahead of the
 //     activations (which come from L2 and land first anyway);
-//   * K slices, where a plan still has them, meet tile by tile: the wavefront that summed a tile
-//     stores its part, waits for its own stores, counts its arrival and, if it is the last,
-//     adds the parts in slice order -- no block-wide barrier in the exchange.
+//   * K slices, where a plan still has them, meet tile by tile without a block-wide barrier: up to
+//     four slices store their parts as their own arrival flags (complemented f32 words in workspace
+//     that is zero between launches) and the last slice's wavefront polls, adds in slice order and
+//     writes the zeros back; plans beyond that count arrivals -- the wavefront that summed a tile
+//     stores its part, waits for its own stores, counts, and the last one adds.
 #include <cstddef>
 
 #include "async_loads.h"
