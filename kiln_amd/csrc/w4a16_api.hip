@@ -489,7 +489,7 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 constexpr int kMidMinM = 33, kMidMinMLongK = 24, kMidMinMLora = 17, kMidMaxM = 128, kMidMaxMSmallest = 320;
 int mid_min_rows(int n, int k, bool lora) {
     // (beyond 68 M weights the two-slab instance leads again: 5120 -> 13824 at 32 rows 23.3 against 25.9 us)
-    return lora ? kMidMinMLora : (k >= 4096 && (long long)k * n <= (68ll << 20) ? kMidMinMLongK : kMidMinM);
+    return lora ? kMidMinMLora : (k >= 4096 && (long long)k * n <= 68000000ll ? kMidMinMLongK : kMidMinM);
 }
 int mid_max_rows(int n, int k) {
     const long long kn = (long long)k * n;
