@@ -128,3 +128,34 @@ def test_replays_of_a_captured_launch_with_the_row_sums_inside(oracle):
             graph.replay()
             torch.cuda.synchronize()
             assert torch.equal(out.view(torch.int16), want.view(torch.int16)), rep
+
+
+def test_fused_swiglu_launch_with_the_row_sums_inside(oracle):
+    """The fused gate+up SwiGLU instance of the kernel takes the same route on a launch of one round
+    (2048 rows, 9216 -> 2 x 1280): equal to the launch in front in every bit, and within the bound of
+    silu(gate) * up formed from the oracle's two f32 GEMMs."""
+    from kiln_amd import marlin_gemm
+    L = _lib.load_tuning()
+    m, k, n_out, g = 2048, 9216, 1280, 128
+    assert L.kiln_w4a16_debug_prefill_rowsum_producers(m, 2 * n_out, k, _cus()) > 0
+    x = oracle.gen_normal_bf16(m, k, 0.5, 77)
+    sides = []
+    for seed in (78, 79):
+        q, s_bits = oracle.np_pack_gptq(oracle.gen_codes(k, n_out, seed)), oracle.gen_scales_f16(k, n_out, g, seed)
+        sides.append((q, s_bits) + tuple(pack.repack_gptq(q, s_bits, None, g)))
+    b_gu, s_gu = pack.interleave_gate_up(sides[0][2], sides[0][3], sides[1][2], sides[1][3], g)
+    bt, st = upload_packed(b_gu, np.asarray(s_gu).view(np.uint16))
+    xt = bf16_tensor(x)
+    try:
+        L.kiln_w4a16_debug_rowsum_fold(0)
+        in_front = marlin_gemm.marlin_w4a16_gemm_swiglu(xt, bt, st, g).clone()
+        L.kiln_w4a16_debug_rowsum_fold(-1)
+        for _ in range(4):
+            assert torch.equal(marlin_gemm.marlin_w4a16_gemm_swiglu(xt, bt, st, g).view(torch.int16), in_front.view(torch.int16))
+    finally:
+        L.kiln_w4a16_debug_rowsum_fold(-1)
+    assert marlin_gemm.workspace_wait_status() == 0
+    gate = oracle.c_w4a16_cpu_path(x, sides[0][0], sides[0][1], g)
+    up = oracle.c_w4a16_cpu_path(x, sides[1][0], sides[1][1], g)
+    err, hv, _ = row_errors(bf16_bits(in_front), oracle.c_swiglu_f32(gate, up), oracle)
+    assert np.all(np.isfinite(hv)) and err.max() <= 1e-2, err.max()
