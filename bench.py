@@ -36,11 +36,11 @@ LAYERS = 16
 TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median replay is reported
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
-# copy (x1.9989 and x1.0): 12307.1 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
+# copy (x1.9989 and x1.0): 12307.4 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25780788, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25781892, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 
@@ -591,8 +591,10 @@ def main() -> int:
         "config": {"workload": "decode MLP projections, M=16: gate+up K=2560->N=18432 then down K=9216->N=2560, "
                                "int4 group-128 weights, fp16 scales, bf16 activations",
                    "m": M, "groupsize": GROUP, "layers_rotated": LAYERS,
-                   "algorithmic_bytes_per_step": bytes_step, "launch": "one HIP graph of all timed steps",
-                   "timed_replays": TIMED_REPLAYS, "statistic": "median replay",
+                   "algorithmic_bytes_per_step": bytes_step,
+                   "launch": "one HIP graph of whole passes of the K timed steps, back to back, replayed per timed region",
+                   "passes_of_k_steps_per_timed_region": replay_log.get("step_passes_of_k_calls_per_timed_region", 1),
+                   "timed_replays": TIMED_REPLAYS, "statistic": "median replay, time per pass of K steps",
                    "wall_ms_per_step": round(wall_step / args.steps * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4),
