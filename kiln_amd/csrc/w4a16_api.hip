@@ -473,24 +473,23 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 }
 
 // Rows the mid-M kernel takes on the automatic plan, from sweeps of the three kernels forced on 13 shapes
-// (the model's, the side-by-side packs, seven of other models) at 20 ... 320 rows.
-// From: 33 rows -- up to 32 the two-slab small-M instance is ahead wherever K = 2560 (gate+up 11.4 against
-// 14.9 us at 32 rows, in-projection 8.2 against 9.1) -- but 24 rows where K >= 4096, whose longer columns the
-// mid-M kernel's K slices and wider products serve better (4096 -> 14336 at 32 rows 17.4 against 21.3 us,
-// 8192 -> 8192 21.8 against 26.3, down projection 11.6 against 12.5; level at 24).  With adapters 17: the
-// two-slab instance needs the projection from a launch in front, the mid-M kernel computes it in its own
-// first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.2 / 12.8 / 16.5 / 16.3 us
-// against 14.4 / 13.3 / 19.2 / 17.0).
+// (the model's, the side-by-side packs, seven of other models) at 17 ... 320 rows.
+// From: 17 rows.  Up to 32 rows it computes one row block of 32 per pass (half the loads of A and half the
+// products of its 64-row pass), and with that it leads the two-slab small-M instance from the first row
+// beyond 16 on every shape (down projection at 17 / 32 rows 8.4 / 9.1 us against 9.7 / 12.5, out-projection
+// 6.4 / 6.7 against 7.8 / 8.4, in-projection 6.6 / 7.2 against 6.7 / 8.4, 4096 -> 14336 12.6 / 13.4 against
+// 15.3 / 21.2) but the wide outputs of a short K, which stay with the two-slab instance up to 32 rows
+// (gate+up 9.8 / 11.4 us against 11.4 / 11.8; 2560 -> 10240 and 12288 level at 32).  With adapters 17
+// everywhere: the two-slab instance needs the projection from a launch in front, the mid-M kernel computes it
+// in its own first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.4 / 10.7 /
+// 13.4 / 13.7 us against 14.4 / 13.3 / 19.2 / 17.0).
 // To: 128 rows (two runs of 64); small weights keep it ahead of the matrix-core kernel's 64-row blocks for
 // longer -- K * N up to 32 M: 192 rows, 256 where K <= 4096 (in-projection at 256 rows 25.2 against 26.5 us,
 // 2560 -> 12288 31.8 against 35.0, down projection at 192 rows 24.5 against 29.1 but 34.5 against 31.3 at 256);
 // up to 12 M: 320 rows (out-projection at 320 rows 16.1 against 23.1, 2560 -> 1024 8.7 against 16.2) -- while
 // on large ones it falls behind from 160 rows on (14336 -> 4096: 55 against 47 us; gate+up 42.5 against 35.2).
-constexpr int kMidMinM = 33, kMidMinMLongK = 24, kMidMinMLora = 17, kMidMaxM = 128, kMidMaxMSmallest = 320;
-int mid_min_rows(int n, int k, bool lora) {
-    // (beyond 68 M weights the two-slab instance leads again: 5120 -> 13824 at 32 rows 23.3 against 25.9 us)
-    return lora ? kMidMinMLora : (k >= 4096 && (long long)k * n <= 68000000ll ? kMidMinMLongK : kMidMinM);
-}
+constexpr int kMidMinM = 17, kMidMinMWideShortK = 33, kMidMaxM = 128, kMidMaxMSmallest = 320;
+int mid_min_rows(int n, int k, bool lora) { return !lora && k < 4096 && n >= 10240 ? kMidMinMWideShortK : kMidMinM; }
 int mid_max_rows(int n, int k) {
     const long long kn = (long long)k * n;
     if (kn <= 12ll << 20) return kMidMaxMSmallest;

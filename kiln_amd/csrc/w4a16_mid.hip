@@ -63,7 +63,8 @@ constexpr int kMidMaxGroups = 4;                // groups per wavefront, at most
 constexpr int kMidFlaggedSlices = kDecodeFlaggedMaxSlices;  // most K slices the counter-free exchange takes
 constexpr int kMidSpinLimit = 1 << 20;          // polls of the other slices' parts before the adding wavefront gives up
 
-// Issue order of a wavefront's loads -- A(g): 16 LDS-direct loads, B(g): NL register loads, the
+// Issue order of a wavefront's loads -- A(g): NA LDS-direct loads (16, or 8 where a run has at most 32
+// rows), B(g): NL register loads, the
 // weights D groups ahead in D + 1 register sets --
 //   before the first step: A(0), B(0) ... B(D-1) (the weights first measured 0.3...0.5 us slower:
 //     loads return in issue order, so A(0) then waits for the weights' trip to memory before the
@@ -75,7 +76,7 @@ struct MidSchedule {
     int wait_a[kMidMaxGroups];
     int wait_b[kMidMaxGroups];
 };
-constexpr MidSchedule mid_schedule(int ng, int nl, int d) {
+constexpr MidSchedule mid_schedule(int ng, int nl, int d, int na) {
     int kind[4 * kMidMaxGroups] = {}, grp[4 * kMidMaxGroups] = {}, size[4 * kMidMaxGroups] = {};
     int n = 0;
     auto push = [&](int k, int g, int sz) {
@@ -93,21 +94,21 @@ constexpr MidSchedule mid_schedule(int ng, int nl, int d) {
         }
         return after;
     };
-    push(0, 0, kMidALoads);
+    push(0, 0, na);
     for (int g = 0; g < d && g < ng; ++g) push(1, g, nl);
     MidSchedule s{};
     for (int g = 0; g < ng; ++g) {
         s.wait_a[g] = issued_after(0, g);
-        if (g + 1 < ng) push(0, g + 1, kMidALoads);
+        if (g + 1 < ng) push(0, g + 1, na);
         if (g + d < ng) push(1, g + d, nl);
         s.wait_b[g] = issued_after(1, g);
     }
     return s;
 }
 
-template <int NG, int NL, int D>
+template <int NG, int NL, int D, int NA>
 struct MidScheduleOf {
-    static constexpr MidSchedule value = mid_schedule(NG, NL, D);
+    static constexpr MidSchedule value = mid_schedule(NG, NL, D, NA);
 };
 
 // The low-rank term of a call with adapters (LORA instances): T = the scaled projection of x onto the
@@ -130,7 +131,9 @@ struct MidLora {
 constexpr int kMidFoldTileWord = 32;  // a copy's words start here (the first words are the small-M kernel's)
 constexpr int kMidFoldSpinLimit = 1 << 20;
 
-template <int TP, int GPW, bool LORA>
+// RBN: row blocks of 32 a pass computes -- 2, or 1 for a launch of at most 32 rows (half the loads of A,
+// fragment reads and products; the other row block's accumulators stay zero and are never stored).
+template <int TP, int GPW, bool LORA, int RBN>
 __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
@@ -210,7 +213,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         const char *base = reinterpret_cast<const char *>(A) + (size_t)(g0 + gi) * 256;
         const uint32_t quad_row = (uint32_t)(lane >> 4) + opaque_zero();  // keeps the offsets below local to this group
 #pragma unroll
-        for (int p = 0; p < kMidALoads; ++p) {
+        for (int p = 0; p < kMidALoads * RBN / 2; ++p) {
             const uint32_t row = 4 * p + quad_row;
             const uint32_t off = min(row, (uint32_t)(M - 1)) * row_pitch + (((uint32_t)(lane & 15) ^ (row & 15)) << 4);
             load_to_lds_b128(base, off, slot_addr + p * 1024);
@@ -262,12 +265,12 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     auto run = [&](auto nc) {
         constexpr int NG = decltype(nc)::value;
         constexpr int NL = 3 * TP;
-        using Sch = MidScheduleOf<NG, NL, D>;
+        using Sch = MidScheduleOf<NG, NL, D, kMidALoads * RBN / 2>;
         request_a(0);
         unrolled<0, (D < NG ? D : NG)>(request_b);
         float s_cur[TP];
         float s_of[NG][TP];   // the scale of every group (this lane's column of each pair)
-        float c_of[NG][2];    // -136 * (sum of the group's activations) of row 32 rb + l32
+        float c_of[NG][RBN];  // -136 * (sum of the group's activations) of row 32 rb + l32
         uint32_t ones;
         asm("s_mov_b32 %0, 0x3f803f80" : "=s"(ones));  // bf16 (1, 1)
         unrolled<0, NG>([&](auto gc) {
@@ -278,9 +281,9 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             wait_vector_loads<Sch::value.wait_a[gi]>();
             if constexpr (gi == 0) KILN_MID_TL(1);  // A(0) has arrived
             if constexpr (gi == 1) KILN_MID_TL(4);  // A(1) has arrived
-            u32x4 af[2][8];
+            u32x4 af[RBN][8];
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
+            for (int rb = 0; rb < RBN; ++rb)
 #pragma unroll
                 for (int s = 0; s < 8; ++s)
                     af[rb][s] = *reinterpret_cast<const u32x4 *>(slot + (rb * 32 + l32) * 256 +
@@ -293,7 +296,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             // 1.0 are exact), two interleaved sums per row block; the lane's half of K here, the other
             // half from lane + 32.
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
+            for (int rb = 0; rb < RBN; ++rb) {
                 float e0 = 0.f, e1 = 0.f;
 #pragma unroll
                 for (int s = 0; s < 7; ++s) {
@@ -324,7 +327,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                 if constexpr (gi > 0) {  // into this group's units: accumulator = sum so far / scale of this group
                     const float f = s_cur[p] * __builtin_amdgcn_rcpf(sn);
 #pragma unroll
-                    for (int rb = 0; rb < 2; ++rb)
+                    for (int rb = 0; rb < RBN; ++rb)
 #pragma unroll
                         for (int r = 0; r < 16; ++r) acc[p][rb][r] *= f;
                 }
@@ -338,7 +341,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                     const uint32_t word = (s >> 1) == 0 ? w4.x : (s >> 1) == 1 ? w4.y : (s >> 1) == 2 ? w4.z : w4.w;
                     const bf16x8 bexp = codes_to_bf16x8(word, dq);
 #pragma unroll
-                    for (int rb = 0; rb < 2; ++rb)
+                    for (int rb = 0; rb < RBN; ++rb)
                         acc[p][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, af[rb][s]), bexp,
                                                                              acc[p][rb], 0, 0, 0);
                 }
@@ -347,7 +350,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
 #pragma unroll
         for (int p = 0; p < TP; ++p)
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
+            for (int rb = 0; rb < RBN; ++rb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) acc[p][rb][r] *= s_cur[p];
         // The B operand carried 136 + d: remove 136 * sum(a) * scale per group by a short extra
@@ -358,9 +361,9 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             constexpr int e = decltype(ec)::value;
             constexpr bool has_odd = 2 * e + 1 < NG;
             constexpr int g_odd = has_odd ? 2 * e + 1 : 2 * e;
-            bf16x8 ax[2];
+            bf16x8 ax[RBN];
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb) {
+            for (int rb = 0; rb < RBN; ++rb) {
                 const float c = h ? (has_odd ? c_of[g_odd][rb] : 0.f) : c_of[2 * e][rb];
                 const uint32_t hi = __builtin_bit_cast(uint32_t, c) & 0xFFFF0000u;
                 const float r1 = c - __builtin_bit_cast(float, hi);                     // exact
@@ -379,7 +382,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
                 const u32x4 r = {pair, pair, pair, 0u};
                 const bf16x8 bx = __builtin_bit_cast(bf16x8, r);
 #pragma unroll
-                for (int rb = 0; rb < 2; ++rb)
+                for (int rb = 0; rb < RBN; ++rb)
                     acc[p][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(ax[rb], bx, acc[p][rb], 0, 0, 0);
             }
         });
@@ -440,9 +443,9 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
             for (int c = wave; c < lo.slices * JS; c += nw) {
                 const int z = c / JS, j8 = (c - z * JS) * 16 + 8 * h;  // this lane's 8 rank columns
                 const bool live_rank = j8 + 8 <= lo.r_total;           // r_total % 8 == 0: all or none
-                u32x4 ta[2], tb[TP];
+                u32x4 ta[RBN], tb[TP];
 #pragma unroll
-                for (int rb = 0; rb < 2; ++rb) {
+                for (int rb = 0; rb < RBN; ++rb) {
                     const int row = zr + min(32 * rb + l32, M - 1);
                     ta[rb] = *reinterpret_cast<const u32x4 *>(lo.t + ((size_t)z * rows + row) * lo.rp + j8);
                 }
@@ -455,7 +458,7 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
 #pragma unroll
                 for (int p = 0; p < TP; ++p)
 #pragma unroll
-                    for (int rb = 0; rb < 2; ++rb)
+                    for (int rb = 0; rb < RBN; ++rb)
                         acc[p][rb] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, ta[rb]),
                                                                              __builtin_bit_cast(bf16x8, tb[p]), acc[p][rb], 0, 0, 0);
             }
@@ -626,9 +629,9 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     }
 }
 
-template <int TP, int GPW>
-hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
-    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora>>(kMidWaves * kMidSlotBytes);
+template <int TP, int GPW, int RBN>
+hipError_t launch_mid_tgr(const MidArgs &a, hipStream_t stream) {
+    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, RBN>>(kMidWaves * kMidSlotBytes);
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
@@ -656,11 +659,17 @@ hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
         }
         grid = dim3(a.lora_producers + col_blocks * a.KS * runs, 1, 1);
     }
-    w4a16_mid_kernel<TP, GPW, kMidLora><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
+    w4a16_mid_kernel<TP, GPW, kMidLora, RBN><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
         a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
         a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0, lo);
     return hipGetLastError();
+}
+
+// at most 32 rows: one row block per pass
+template <int TP, int GPW>
+hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
+    return a.M <= 32 ? launch_mid_tgr<TP, GPW, 1>(a, stream) : launch_mid_tgr<TP, GPW, 2>(a, stream);
 }
 
 template <int TP>

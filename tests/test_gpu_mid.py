@@ -31,6 +31,21 @@ def test_mid_rows_on_the_model_shapes(oracle, m, k, n):
     _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
 
 
+@pytest.mark.parametrize("m", [17, 25, 32])
+@pytest.mark.parametrize("k,n", MODEL_SHAPES)
+def test_one_row_block_per_pass_on_the_model_shapes(oracle, m, k, n):
+    """17...32 rows: the kernel computes one row block of 32 per pass (half the loads of A and half the
+    products).  The automatic dispatch sends every shape there but the widest output of the shortest K;
+    forced through the tuning build all four run it."""
+    L = _lib.load_tuning()
+    assert _takes_mid(_lib.load(), m, n, k) == ((k, n) != (2560, 18432))
+    L.kiln_w4a16_debug_mid(1, 0, 0)
+    assert _takes_mid(L, m, n, k)
+    x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=3 * m + n)
+    b, s = pack.repack_gptq(q, s_bits, None, 128)
+    _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
+
+
 def _mid_instances():
     cases = []
     for pairs in (1, 2, 3):
@@ -56,7 +71,7 @@ def test_every_mid_instance(oracle, pairs, gs, ks):
     x, q, s_bits = oracle.gen_problem(100, k, n, 128, seed=pairs * 1000 + gs * 10 + ks)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
     L.kiln_w4a16_debug_mid(1, pairs, ks)
-    for m in (5, 64, 100):
+    for m in (5, 32, 64, 100):       # up to 32 rows: the instances that compute one row block per pass
         assert _takes_mid(L, m, n, k), (m, k, n)
         _run_case(oracle, m, k, n, 128, x[:m], b, s, q, s_bits)
 

@@ -56,10 +56,11 @@ def test_sixteen_wavefronts_only_where_twelve_cannot_form_the_plan():
 
 
 @pytest.mark.parametrize("m,k,n,want", [
-    # from: 33 rows, 24 on long K up to 68 M weights
-    (32, 2560, 18432, "small"), (33, 2560, 18432, "mid"), (32, 2560, 8192, "small"),
-    (23, 4096, 4096, "small"), (24, 4096, 4096, "mid"), (24, 9216, 2560, "mid"), (32, 8192, 8192, "mid"),
-    (32, 5120, 13824, "small"),
+    # from: 17 rows; wide outputs of a short K stay with the two-slab small-M instance up to 32 rows
+    (16, 9216, 2560, "small"), (17, 9216, 2560, "mid"), (17, 4096, 2560, "mid"), (17, 2560, 8192, "mid"),
+    (17, 2560, 1024, "mid"), (24, 4096, 4096, "mid"), (32, 8192, 8192, "mid"), (32, 5120, 13824, "mid"),
+    (17, 2560, 18432, "small"), (32, 2560, 18432, "small"), (33, 2560, 18432, "mid"), (32, 2560, 10240, "small"),
+    (32, 3584, 18944, "small"),
     # to: 128 rows; 192 / 256 / 320 on small weights
     (128, 2560, 18432, "mid"), (129, 2560, 18432, "matrix-core"), (160, 14336, 4096, "matrix-core"),
     (160, 8192, 8192, "matrix-core"),
