@@ -131,13 +131,14 @@ struct MidLora {
 constexpr int kMidFoldTileWord = 32;  // a copy's words start here (the first words are the small-M kernel's)
 constexpr int kMidFoldSpinLimit = 1 << 20;
 
-// RBN: row blocks of 32 a pass computes -- 2, or 1 for a launch of at most 32 rows (half the loads of A,
-// fragment reads and products; the other row block's accumulators stay zero and are never stored).
+// The work of one block.  RBN: row blocks of 32 its pass computes -- 2, or 1 where the block's run of rows
+// has at most 32 (a launch of up to 32 rows, or the last run of a longer one: half the loads of A, fragment
+// reads and products; the other row block's accumulators stay zero and are never stored).
 template <int TP, int GPW, bool LORA, int RBN>
-__global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
+__device__ __forceinline__ void mid_block(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
-    int GS, int full_waves, int swiglu, int flagged, int col_shift, MidLora lo) {
+    int GS, int full_waves, int swiglu, int flagged, int col_shift, const MidLora &lo) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     __shared__ int s_last;
     const int tid = threadIdx.x;
@@ -629,9 +630,39 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     }
 }
 
-template <int TP, int GPW, int RBN>
-hipError_t launch_mid_tgr(const MidArgs &a, hipStream_t stream) {
-    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, RBN>>(kMidWaves * kMidSlotBytes);
+// SHORT: the launch has at most 32 rows (one row block per pass, and a kernel with as few registers as that
+// takes: a launch costs more the more registers its wavefronts hold, 0.3 us here); otherwise every block
+// looks at its own run of rows -- the last run of a launch may have 32 or fewer.
+template <int TP, int GPW, bool LORA, bool SHORT>
+__global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
+    const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
+    uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
+    int GS, int full_waves, int swiglu, int flagged, int col_shift, MidLora lo) {
+    if constexpr (SHORT) {
+        mid_block<TP, GPW, LORA, 1>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS, full_waves, swiglu,
+                                    flagged, col_shift, lo);
+    } else {
+        // the run of 64 rows this block belongs to, as mid_block maps its index (a producer block of a call
+        // with adapters belongs to none: either instance runs the projection and returns)
+        int bz = blockIdx.z;
+        if constexpr (LORA) {
+            if (lo.producers > 0) {
+                const int id = (int)blockIdx.x - lo.producers;
+                bz = id < 0 ? 0 : id / lo.col_blocks / KS;
+            }
+        }
+        if (rows - bz * kMidRows <= 32)
+            mid_block<TP, GPW, LORA, 1>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS, full_waves,
+                                        swiglu, flagged, col_shift, lo);
+        else
+            mid_block<TP, GPW, LORA, 2>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS, full_waves,
+                                        swiglu, flagged, col_shift, lo);
+    }
+}
+
+template <int TP, int GPW, bool SHORT>
+hipError_t launch_mid_tgs(const MidArgs &a, hipStream_t stream) {
+    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, SHORT>>(kMidWaves * kMidSlotBytes);
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
@@ -659,17 +690,16 @@ hipError_t launch_mid_tgr(const MidArgs &a, hipStream_t stream) {
         }
         grid = dim3(a.lora_producers + col_blocks * a.KS * runs, 1, 1);
     }
-    w4a16_mid_kernel<TP, GPW, kMidLora, RBN><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
+    w4a16_mid_kernel<TP, GPW, kMidLora, SHORT><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
         a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
         a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0, lo);
     return hipGetLastError();
 }
 
-// at most 32 rows: one row block per pass
 template <int TP, int GPW>
 hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
-    return a.M <= 32 ? launch_mid_tgr<TP, GPW, 1>(a, stream) : launch_mid_tgr<TP, GPW, 2>(a, stream);
+    return a.M <= 32 ? launch_mid_tgs<TP, GPW, true>(a, stream) : launch_mid_tgs<TP, GPW, false>(a, stream);
 }
 
 template <int TP>
