@@ -40,7 +40,7 @@ TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median rep
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25781463, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25781507, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 
@@ -111,11 +111,12 @@ def other_configurations(torch, marlin_gemm, dev, make_layer, timed_graph, shape
     # the same adapters on a decode step's 16 rows (small-M kernels with the low-rank term)
     us = time_shape(16, 2560, 18432, 200, lora=(la, lb, ranks, lscales))
     extra["m16_gate_up_lora_r16_r32"] = {"us": round(us, 2)}
-    # cfg 3: every quantised linear of a 32-layer model, one decode step, M in {1, 4, 16, 64}
+    # cfg 3: every quantised linear of a 32-layer model, one decode step, M in {1, 4, 16, 64} (and 32, which the
+    # configuration does not name: the row count at which the mid-M kernel's one-row-block pass runs)
     sweep_shapes = [(2560, 8192), (4096, 2560), (2560, 18432), (9216, 2560)]
     sweep_w = [[make_layer(k, n) for (k, n) in sweep_shapes] for _ in range(32)]
     w_bytes = 32 * sum(k * n // 2 + (k // GROUP) * n * 2 for (k, n) in sweep_shapes)
-    for m_sw in (1, 4, 16, 64):
+    for m_sw in (1, 4, 16, 32, 64):
         xs = [torch.randn(m_sw, k, device=dev).to(torch.bfloat16) for (k, n) in sweep_shapes]
         os_ = [torch.empty(m_sw, n, dtype=torch.bfloat16, device=dev) for (k, n) in sweep_shapes]
         def sweep(_i):

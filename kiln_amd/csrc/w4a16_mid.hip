@@ -138,13 +138,12 @@ template <int TP, int GPW, bool LORA, int RBN>
 __device__ __forceinline__ void mid_block(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
-    int GS, int full_waves, int swiglu, int flagged, int col_shift, const MidLora &lo) {
+    int GS, int full_waves, int swiglu, int flagged, int col_shift, const MidLora &lo, int nw) {
     extern __shared__ __attribute__((aligned(1024))) unsigned char lds[];
     __shared__ int s_last;
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int nw = blockDim.x >> 6;
     const int l32 = lane & 31, h = lane >> 5;
     const int G = K / kGroupK;
 #ifdef KILN_MID_TIMELINE
@@ -630,17 +629,26 @@ __device__ __forceinline__ void mid_block(
     }
 }
 
-// SHORT: the launch has at most 32 rows (one row block per pass, and a kernel with as few registers as that
-// takes: a launch costs more the more registers its wavefronts hold, 0.3 us here); otherwise every block
-// looks at its own run of rows -- the last run of a launch may have 32 or fewer.
-template <int TP, int GPW, bool LORA, bool SHORT>
+// Which row blocks a launch's blocks pass over, a kernel for each so that none carries code or registers it
+// does not use (a launch costs more the more registers its wavefronts hold, 0.3 us between the first and
+// the second here, and the kernel with both bodies measured 0.5 us above the second at 64 rows):
+// kMidOneRowBlock -- at most 32 rows in the launch; kMidTwoRowBlocks -- every run of 64 rows has more
+// than 32; kMidRowBlocksByRun -- the last run has 32 or fewer and the runs before it 64, each block looks
+// at its own.
+constexpr int kMidOneRowBlock = 1, kMidTwoRowBlocks = 2, kMidRowBlocksByRun = 0;
+
+template <int TP, int GPW, bool LORA, int ROW_BLOCKS>
 __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
     int GS, int full_waves, int swiglu, int flagged, int col_shift, MidLora lo) {
-    if constexpr (SHORT) {
-        mid_block<TP, GPW, LORA, 1>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS, full_waves, swiglu,
-                                    flagged, col_shift, lo);
+    // the block's wavefronts, read here: in the kernel itself the compiler knows every block to be whole
+    // and reads the launch's block size, in a device function it first asks whether this block is a partial
+    // one (a dependent load at the very start)
+    const int nw = blockDim.x >> 6;
+    if constexpr (ROW_BLOCKS != kMidRowBlocksByRun) {
+        mid_block<TP, GPW, LORA, ROW_BLOCKS>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS,
+                                             full_waves, swiglu, flagged, col_shift, lo, nw);
     } else {
         // the run of 64 rows this block belongs to, as mid_block maps its index (a producer block of a call
         // with adapters belongs to none: either instance runs the projection and returns)
@@ -653,16 +661,16 @@ __global__ __launch_bounds__(kMidWaves * 64) void w4a16_mid_kernel(
         }
         if (rows - bz * kMidRows <= 32)
             mid_block<TP, GPW, LORA, 1>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS, full_waves,
-                                        swiglu, flagged, col_shift, lo);
+                                        swiglu, flagged, col_shift, lo, nw);
         else
             mid_block<TP, GPW, LORA, 2>(A_all, B, S, C_all, partial_all, counters_all, rows, N, K, Gs, KS, GS, full_waves,
-                                        swiglu, flagged, col_shift, lo);
+                                        swiglu, flagged, col_shift, lo, nw);
     }
 }
 
-template <int TP, int GPW, bool SHORT>
+template <int TP, int GPW, int ROW_BLOCKS>
 hipError_t launch_mid_tgs(const MidArgs &a, hipStream_t stream) {
-    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, SHORT>>(kMidWaves * kMidSlotBytes);
+    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, ROW_BLOCKS>>(kMidWaves * kMidSlotBytes);
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
@@ -690,7 +698,7 @@ hipError_t launch_mid_tgs(const MidArgs &a, hipStream_t stream) {
         }
         grid = dim3(a.lora_producers + col_blocks * a.KS * runs, 1, 1);
     }
-    w4a16_mid_kernel<TP, GPW, kMidLora, SHORT><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
+    w4a16_mid_kernel<TP, GPW, kMidLora, ROW_BLOCKS><<<grid, a.waves * 64, a.waves * kMidSlotBytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, a.partial, a.counters, a.M,
         a.N, a.K, a.Gs, a.KS, a.GS, full_waves, a.swiglu ? 1 : 0, a.flagged ? 1 : 0,
         a.flagged ? exchange_column_shift((NT + 2 * TP - 1) / (2 * TP)) : 0, lo);
@@ -699,7 +707,10 @@ hipError_t launch_mid_tgs(const MidArgs &a, hipStream_t stream) {
 
 template <int TP, int GPW>
 hipError_t launch_mid_tg(const MidArgs &a, hipStream_t stream) {
-    return a.M <= 32 ? launch_mid_tgs<TP, GPW, true>(a, stream) : launch_mid_tgs<TP, GPW, false>(a, stream);
+    if (a.M <= 32) return launch_mid_tgs<TP, GPW, kMidOneRowBlock>(a, stream);
+    const int last_run = a.M - (a.M - 1) / kMidRows * kMidRows;
+    return last_run <= 32 ? launch_mid_tgs<TP, GPW, kMidRowBlocksByRun>(a, stream)
+                          : launch_mid_tgs<TP, GPW, kMidTwoRowBlocks>(a, stream);
 }
 
 template <int TP>

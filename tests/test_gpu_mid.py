@@ -71,7 +71,9 @@ def test_every_mid_instance(oracle, pairs, gs, ks):
     x, q, s_bits = oracle.gen_problem(100, k, n, 128, seed=pairs * 1000 + gs * 10 + ks)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
     L.kiln_w4a16_debug_mid(1, pairs, ks)
-    for m in (5, 32, 64, 100):       # up to 32 rows: the instances that compute one row block per pass
+    # three kernels per instance: one row block per pass (up to 32 rows), two (every run of 64 has more
+    # than 32), and the choice by run (80 rows: a run of 64 and one of 16)
+    for m in (5, 32, 64, 80, 100):
         assert _takes_mid(L, m, n, k), (m, k, n)
         _run_case(oracle, m, k, n, 128, x[:m], b, s, q, s_bits)
 
