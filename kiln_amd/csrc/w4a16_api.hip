@@ -511,11 +511,16 @@ bool mid_flagged(const MidArgs &a) {
 // parallelism for L2 traffic); a launch costs about 4.5 us beside its rounds of blocks, an exchange
 // between K slices through counters 1.5 us at two slices and 1.7 us more per further slice
 // (out-projection at 64 rows: 11.5 us unsliced, 10.4 in two slices, 13.8 in four), the counter-free
-// exchange 1 us less (9.4 in two slices).  Every round of blocks after the first costs its start on top
-// (2 us: without it many rounds of short slices looked cheap -- 5120 -> 13824 at 128 rows 58 us in five
-// slices against 48 in two).  Checked against every forced plan on 20 shapes (those four, the
-// side-by-side packs and 14 of other models) at 40, 64, 96 and 128 rows: the plan picked is 1.6 %
-// slower than the best on average, 25 % at worst (4096 -> 1024, where four slices would beat two).
+// exchange 1 us less at two slices (9.4) and 0.5 us per further slice (the four-slice figure above held a
+// second round of blocks; 4096 -> 1024, 128 blocks in four slices: 6.4 us at 64 rows against 7.9 in two).
+// Every round of blocks after the first costs its start on top (2 us: without it many rounds of short
+// slices looked cheap -- 5120 -> 13824 at 128 rows 58 us in five slices against 48 in two).  Checked
+// against every forced plan on 22 shapes (those four, the side-by-side packs and 16 of other models) at
+// 17, 32, 40, 64, 96 and 128 rows: the plan picked is 0.4 % slower than the best on average from 40 rows
+// on and 1.3 % at 17 and 32, 10 % at worst where the automatic route takes this kernel (3584 -> 18944 at
+// 40 rows, 4096 -> 11008 at 17: three pairs in two slices where two pairs unsliced would lead).  Eight
+// narrow outputs of a long K swept afterwards (4096 -> 512 ... 8192 -> 3072 at 24, 64 and 128 rows): within
+// 4 % of the best plan but on 6144 -> 1536 (6...12 %: 12 groups dealt to 8 wavefronts count as 16).
 MidPlan plan_mid(int m, int n, int k, int cus) {
     MidPlan best;
     const int G = k / kGroupK, runs = ceil_div(m, mid_max_rows_per_run());
@@ -535,7 +540,7 @@ MidPlan plan_mid(int m, int n, int k, int cus) {
             const int col_blocks = mid_column_blocks(a);
             if ((size_t)runs * col_blocks * sizeof(int) > kCounterCapacity) continue;
             const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
-            const float exchange = ks == 1 ? 0.f : (mid_flagged(a) ? 1.7f * ks - 2.9f : 1.7f * ks - 1.9f);
+            const float exchange = ks == 1 ? 0.f : (mid_flagged(a) ? 0.5f * ks - 0.5f : 1.7f * ks - 1.9f);
             const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange + 2.0f * (rounds - 1);
             if (!best.ok || cost < best.cost) {
                 best.ok = true;

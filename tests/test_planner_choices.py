@@ -76,6 +76,8 @@ def test_which_kernel_takes_a_row_count(m, k, n, want):
     (64, 2560, 8192, (1, 1)), (64, 4096, 2560, (1, 2)), (64, 2560, 18432, (3, 1)), (64, 9216, 2560, (1, 3)),
     # rounds after the first cost their start: no pile of short slices
     (128, 5120, 13824, (3, 2)), (96, 3584, 18944, (2, 1)), (128, 3584, 18944, (2, 1)),
+    # one round either way: four short slices through the counter-free exchange lead two long ones
+    (64, 4096, 1024, (1, 4)), (17, 4096, 1024, (1, 4)), (128, 4096, 1024, (1, 4)),
 ])
 def test_mid_m_plans(m, k, n, want):
     assert _route(m, k, n) == ("mid",) + want
