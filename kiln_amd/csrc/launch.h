@@ -24,9 +24,9 @@ constexpr size_t kWsFoldFlagOffset = kWsCounterBytes + kWsFlaggedBytes - kWsFold
 constexpr size_t kWsZeroedBytes = kWsCounterBytes + kWsFlaggedBytes;
 enum WaitGaveUp : unsigned {
     kGaveUpDecodeExchange = 1u,  // K slices of a launch of up to 16 rows
-    kGaveUpMidExchange = 2u,     // K slices of a launch of 33...192 rows
+    kGaveUpMidExchange = 2u,     // K slices of a launch of 17...320 rows
     kGaveUpDecodeFold = 4u,      // a block of up to 16 rows waiting for the folded LoRA projection
-    kGaveUpMidFold = 8u,         // the same at 17...192 rows
+    kGaveUpMidFold = 8u,         // the same at 17...320 rows
     kGaveUpPrefillFold = 16u,    // the same on the matrix-core path
 };
 

@@ -505,7 +505,7 @@ bool mid_flagged(const MidArgs &a) {
 }
 
 // Plan for the mid-M kernel: pairs of tiles per block, K slices, wavefronts.  Cost in microseconds,
-// fitted to a sweep of the four projection shapes at 33...192 rows: a wavefront's group step is
+// fitted to a sweep of the four projection shapes at 33...192 rows (and checked from 17 on, see below): a wavefront's group step is
 // bound by the round trip of its activations through L2 and by the products of its pairs
 // (0.75 + 0.55 us per pair; every block re-reads its rows of A, so fewer and wider blocks trade
 // parallelism for L2 traffic); a launch costs about 4.5 us beside its rounds of blocks, an exchange
@@ -570,8 +570,9 @@ MidArgs mid_args(const MidPlan &mp, int m, int n, int k) {
 
 void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lora, GemmPlan *gp) {
     *gp = GemmPlan{};
-    // 33...128 rows: the mid-M kernel, one pass over the weights per 64 rows (with adapters whose
-    // stacked rank is a multiple of 8: the low-rank term is added from a projection launched in front)
+    // mid_min_rows() ... mid_max_rows() rows: the mid-M kernel, one pass over the weights per 64 rows (with
+    // adapters whose stacked rank is a multiple of 8: the low-rank term is added from a projection that runs
+    // in the launch's first blocks where it fits, else from one launched in front)
     // (a call pinned to a block shape of the matrix-core kernel goes there)
     const bool prefill_pinned = g_tune.prefill_bm != 0 || g_tune.prefill_bn != 0 || g_tune.prefill_ks != 0 || g_tune.prefill_nb_full >= 0;
     if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&

@@ -3,10 +3,11 @@
 // Covers the row counts between the decode kernels (one or two 16-row slabs, 16x16x32
 // products) and the prefill kernel (whole-chip tiling, matrix-core bound): the arm of the
 // reference dispatcher that pads M to 16 * thread_m_blocks up to 64 rows
-// (crates/kiln-marlin-gemm/csrc/marlin_kernel.cu:784-816).  At 33...128 rows the problem is
-// still bound by the int4 weight stream, but the products are no longer free: 64 rows take
-// v_mfma_f32_32x32x16_bf16 (the 16-row shape runs at half the rate per flop) and one pass over
-// the weights.
+// (crates/kiln-marlin-gemm/csrc/marlin_kernel.cu:784-816).  At 17...128 rows (and up to 320 on
+// small weights) the problem is still bound by the int4 weight stream, but the products are no
+// longer free: a run of 64 rows takes v_mfma_f32_32x32x16_bf16 (the 16-row shape runs at half the
+// rate per flop) and one pass over the weights; a run of up to 32 rows computes one of the two row
+// blocks only.
 //
 // Work split (group-major, as in the decode kernels): a block owns TP pairs of neighbouring
 // 16-column tiles (32 columns per pair = one 32x32 product tile) and one K slice of GS groups;
