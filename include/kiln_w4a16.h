@@ -314,6 +314,28 @@ const char *kiln_w4a16_status_string(kiln_marlin_status_t status);
 /* Layout revision written into persisted artefacts; bumps when the tile layout changes. */
 int kiln_w4a16_layout_version(void);
 
+/*
+ * Plan queries: what the library would run for a plain GEMM of these sizes on a part with `cus`
+ * compute units.  Pure host functions (no GPU is touched, nothing is launched); they exist for
+ * benchmarks, profiles and tests that must name the kernel they measure, and have no counterpart in
+ * the reference (whose one kernel picks its tile from a fixed table, marlin_kernel.cu:784-816).
+ * The numbers describe this library's kernels and may change with any revision.
+ *
+ * kiln_w4a16_debug_gemm_plan: out[8] = {matrix-core kernel?, launches of the small-M kernels, block
+ *   rows, block columns, whole column blocks, K slices (the last four of the matrix-core kernel),
+ *   mid-M kernel?, its tile pairs per block * 16 + K slices}.  Returns 0, or 1 for sizes no kernel takes.
+ * kiln_w4a16_debug_decode_plan: the small-M plan for one run of m <= 32 rows, out[8] = {K slices,
+ *   groups per slice, chunks per wavefront, blocks per slice, wavefronts per block, fragments straight
+ *   from L2?, register-fragment instance?, tiles per block (negative: the private-staging instance)}.
+ *   Returns 0, or 1 if no plan fits.
+ * kiln_w4a16_debug_prefill_rowsum_producers: where the matrix-core kernel's row sums come from:
+ *   > 0 that many blocks of the product's own launch, 0 a launch in front, -2 every block sums its own
+ *   rows, -3 another kernel takes the call, -1 bad sizes.
+ */
+int kiln_w4a16_debug_gemm_plan(int prob_m, int prob_n, int prob_k, int cus, int *out);
+int kiln_w4a16_debug_decode_plan(int prob_m, int prob_n, int prob_k, int cus, int *out);
+int kiln_w4a16_debug_prefill_rowsum_producers(int prob_m, int prob_n, int prob_k, int cus);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,6 +36,9 @@ EXPORTS = (
     "kiln_w4a16_unpack_to_gptq",
     "kiln_w4a16_status_string",
     "kiln_w4a16_layout_version",
+    "kiln_w4a16_debug_gemm_plan",
+    "kiln_w4a16_debug_decode_plan",
+    "kiln_w4a16_debug_prefill_rowsum_producers",
 )
 
 # every symbol include/kiln_marlin_proj.h declares

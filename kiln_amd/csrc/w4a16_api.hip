@@ -1048,7 +1048,7 @@ kiln_marlin_status_t kiln_w4a16_workspace_reset(void *workspace, void *stream) {
 }
 
 // The small-M plan for a run of m rows on a part with `cus` compute units (a pure query, no GPU
-// needed; not part of the public header): out = {KS, GS, U, BPS, waves, direct, regs, gm_tiles}.
+// needed): out = {KS, GS, U, BPS, waves, direct, regs, gm_tiles}.
 // m <= 32; returns 0, or 1 if no plan fits.
 int kiln_w4a16_debug_decode_plan(int m, int n, int k, int cus, int *out) {
     if (m < 1 || m > 32 || cus < 1 || !shape_ok(n, k, 128)) return 1;
@@ -1062,7 +1062,7 @@ int kiln_w4a16_debug_decode_plan(int m, int n, int k, int cus, int *out) {
     return 0;
 }
 
-// Which path a plain GEMM takes (a pure query, not part of the public header):
+// Which path a plain GEMM takes (a pure query):
 // out = {matrix-core path?, small-M launches, block rows, block columns, whole column blocks, K slices,
 //        mid-M kernel?, its tile pairs * 16 + K slices}.
 int kiln_w4a16_debug_gemm_plan(int m, int n, int k, int cus, int *out) {
