@@ -69,15 +69,17 @@ constexpr int kMidSpinLimit = 1 << 20;          // polls of the other slices' pa
 // weights D groups ahead in D + 1 register sets --
 //   before the first step: A(0), B(0) ... B(D-1) (the weights first measured 0.3...0.5 us slower:
 //     loads return in issue order, so A(0) then waits for the weights' trip to memory before the
-//     fragments can be read and A(1) asked for);
-//   step g: [wait for A(g)] fragments to registers, A(g+1), B(g+D), [wait for B(g)], products.
+//     fragments can be read and A(1) asked for), A(1) ... A(DA-1);
+//   step g: [wait for A(g)] fragments to registers, A(g+DA), B(g+D), [wait for B(g)], products.
+// DA = groups of A in flight: 1 where a group fills the wavefront's slot (64 rows), 2 where it fills half
+// (one row block per pass: the halves take turns).
 // wait_a[g] / wait_b[g] = loads issued after A(g) / B(g) up to that wait: what may still be
 // outstanding when the wait returns.
 struct MidSchedule {
     int wait_a[kMidMaxGroups];
     int wait_b[kMidMaxGroups];
 };
-constexpr MidSchedule mid_schedule(int ng, int nl, int d, int na) {
+constexpr MidSchedule mid_schedule(int ng, int nl, int d, int na, int da) {
     int kind[4 * kMidMaxGroups] = {}, grp[4 * kMidMaxGroups] = {}, size[4 * kMidMaxGroups] = {};
     int n = 0;
     auto push = [&](int k, int g, int sz) {
@@ -97,19 +99,20 @@ constexpr MidSchedule mid_schedule(int ng, int nl, int d, int na) {
     };
     push(0, 0, na);
     for (int g = 0; g < d && g < ng; ++g) push(1, g, nl);
+    for (int g = 1; g < da && g < ng; ++g) push(0, g, na);
     MidSchedule s{};
     for (int g = 0; g < ng; ++g) {
         s.wait_a[g] = issued_after(0, g);
-        if (g + 1 < ng) push(0, g + 1, na);
+        if (g + da < ng) push(0, g + da, na);
         if (g + d < ng) push(1, g + d, nl);
         s.wait_b[g] = issued_after(1, g);
     }
     return s;
 }
 
-template <int NG, int NL, int D, int NA>
+template <int NG, int NL, int D, int NA, int DA>
 struct MidScheduleOf {
-    static constexpr MidSchedule value = mid_schedule(NG, NL, D, NA);
+    static constexpr MidSchedule value = mid_schedule(NG, NL, D, NA, DA);
 };
 
 // The low-rank term of a call with adapters (LORA instances): T = the scaled projection of x onto the
@@ -210,6 +213,7 @@ __device__ __forceinline__ void mid_block(
     unsigned char *slot = lds + wave * kMidSlotBytes;
     const unsigned slot_addr = (unsigned)(size_t)(lds_ptr_t)slot;
     const uint32_t row_pitch = (uint32_t)K * 2;
+    constexpr int kASlots = RBN == 1 ? 2 : 1;  // groups of A a slot holds, and as many are in flight
     auto request_a = [&](int gi) {
         const char *base = reinterpret_cast<const char *>(A) + (size_t)(g0 + gi) * 256;
         const uint32_t quad_row = (uint32_t)(lane >> 4) + opaque_zero();  // keeps the offsets below local to this group
@@ -217,7 +221,7 @@ __device__ __forceinline__ void mid_block(
         for (int p = 0; p < kMidALoads * RBN / 2; ++p) {
             const uint32_t row = 4 * p + quad_row;
             const uint32_t off = min(row, (uint32_t)(M - 1)) * row_pitch + (((uint32_t)(lane & 15) ^ (row & 15)) << 4);
-            load_to_lds_b128(base, off, slot_addr + p * 1024);
+            load_to_lds_b128(base, off, slot_addr + (uint32_t)(gi % kASlots) * (kMidSlotBytes / 2) + p * 1024);
         }
     };
 
@@ -266,9 +270,10 @@ __device__ __forceinline__ void mid_block(
     auto run = [&](auto nc) {
         constexpr int NG = decltype(nc)::value;
         constexpr int NL = 3 * TP;
-        using Sch = MidScheduleOf<NG, NL, D, kMidALoads * RBN / 2>;
+        using Sch = MidScheduleOf<NG, NL, D, kMidALoads * RBN / 2, kASlots>;
         request_a(0);
         unrolled<0, (D < NG ? D : NG)>(request_b);
+        if constexpr (kASlots == 2 && NG > 1) request_a(1);
         float s_cur[TP];
         float s_of[NG][TP];   // the scale of every group (this lane's column of each pair)
         float c_of[NG][RBN];  // -136 * (sum of the group's activations) of row 32 rb + l32
@@ -287,10 +292,10 @@ __device__ __forceinline__ void mid_block(
             for (int rb = 0; rb < RBN; ++rb)
 #pragma unroll
                 for (int s = 0; s < 8; ++s)
-                    af[rb][s] = *reinterpret_cast<const u32x4 *>(slot + (rb * 32 + l32) * 256 +
-                                                                 (((2 * s + h) ^ (l32 & 15)) << 4));
-            wait_lds_reads();  // the slot is free again
-            if constexpr (gi + 1 < NG) request_a(gi + 1);
+                    af[rb][s] = *reinterpret_cast<const u32x4 *>(slot + (gi % kASlots) * (kMidSlotBytes / 2) +
+                                                                 (rb * 32 + l32) * 256 + (((2 * s + h) ^ (l32 & 15)) << 4));
+            wait_lds_reads();  // the slot (or this half of it) is free again
+            if constexpr (gi + kASlots < NG) request_a(gi + kASlots);
             if constexpr (gi + D < NG) request_b(std::integral_constant<int, gi + D>{});
             // Row sums of the group for the offset term, on the vector unit while the matrix unit
             // multiplies: v_dot2c_f32_bf16 adds both halves of a register to an f32 sum (products with
