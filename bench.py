@@ -40,7 +40,7 @@ TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median rep
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25781507, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25781652, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 
@@ -292,7 +292,7 @@ def main() -> int:
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extra", action="store_true",
                     help="skip the legs reported under `extra` (every launch is then an M=16 launch of the workload)")
-    ap.add_argument("--profile", choices=["decode", "decode_m1", "mid", "prefill", "lora", "pack"], default=None,
+    ap.add_argument("--profile", choices=["decode", "decode_m1", "mid", "mid_m32", "prefill", "lora", "pack"], default=None,
                     help="for rocprofv3: launch K eager steps of the chosen regime (no graph, no CPU "
                          "baseline, no extra legs) plus one 64 MiB device copy that calibrates the "
                          "memory-traffic counters, print no JSON; prefill: the two cfg 2 GEMMs at M=2048, "
@@ -365,11 +365,12 @@ def main() -> int:
                     b, s = layers[i % LAYERS][name]
                     marlin_gemm.marlin_w4a16_gemm(x1[name], b, s, GROUP, out=o1[name])
                 marlin_gemm.marlin_w4a16_gemm(xs, sq[i % LAYERS][0], sq[i % LAYERS][1], GROUP, out=os_)
-        elif args.profile == "mid":
-            sweep = {"in_proj": (2560, 8192), "out_proj": (4096, 2560), **shapes}
+        elif args.profile in ("mid", "mid_m32"):
+            rows = 64 if args.profile == "mid" else 32   # 32: the mid-M kernel's one-row-block pass (gate+up at 32 rows
+            sweep = {"in_proj": (2560, 8192), "out_proj": (4096, 2560), **shapes}   # takes the two-slab small-M instance)
             sw = {name: [make_layer(*kn) for _ in range(8)] for name, kn in sweep.items() if name not in shapes}
-            x64 = {name: torch.randn(64, kn[0], device=dev).to(torch.bfloat16) for name, kn in sweep.items()}
-            o64 = {name: torch.empty(64, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in sweep.items()}
+            x64 = {name: torch.randn(rows, kn[0], device=dev).to(torch.bfloat16) for name, kn in sweep.items()}
+            o64 = {name: torch.empty(rows, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in sweep.items()}
             for i in range(args.steps):
                 for name in sweep:
                     b, s = layers[i % LAYERS][name] if name in shapes else sw[name][i % 8]

@@ -137,7 +137,8 @@ constexpr int kMidFoldSpinLimit = 1 << 20;
 
 // The work of one block.  RBN: row blocks of 32 its pass computes -- 2, or 1 where the block's run of rows
 // has at most 32 (a launch of up to 32 rows, or the last run of a longer one: half the loads of A, fragment
-// reads and products; the other row block's accumulators stay zero and are never stored).
+// reads and products; the other row block's accumulators stay zero, and its items take no part in the
+// wavefronts' meeting, in the exchange between K slices or in the store).
 template <int TP, int GPW, bool LORA, int RBN>
 __device__ __forceinline__ void mid_block(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
@@ -525,7 +526,7 @@ __device__ __forceinline__ void mid_block(
 #pragma unroll
         for (int p = p0; p < p1; ++p)
 #pragma unroll
-            for (int rb = 0; rb < 2; ++rb)
+            for (int rb = 0; rb < RBN; ++rb)  // (one row block per pass: nobody reads the other one's items below)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
                     mine[(((p - p0) * 2 + rb) * 4 + q) * 64 + lane] =
@@ -533,6 +534,7 @@ __device__ __forceinline__ void mid_block(
         __syncthreads();
         if constexpr (p0 == 0) KILN_MID_TL(6);  // every wavefront's tiles are in LDS
         if (flagged) {  // eight wavefronts: item (p0 + j) * 8 + wave for each pair j of the phase
+            if (RBN == 1 && wave >= 4) return;  // items of the row block this pass does not compute
 #pragma unroll
             for (int j = 0; j < p1 - p0; ++j) {
                 const int item = (p0 + j) * 8 + wave;
@@ -548,6 +550,7 @@ __device__ __forceinline__ void mid_block(
             return;
         }
         for (int item = p0 * 8 + wave; item < p1 * 8; item += nw) {
+            if (RBN == 1 && (item & 4)) continue;  // an item of the row block this pass does not compute
             const f32x4 sum = sum_over_wavefronts(item - p0 * 8);
             if (KS == 1) {
                 store_item(sum, item);
@@ -567,7 +570,7 @@ __device__ __forceinline__ void mid_block(
         // it waits for is running or done.  Each part is loaded once per poll; the loads are
         // straight-line code up to their wait, so the parts of absent slices (zeros nobody
         // writes, or another run's parts) are loaded too and ignored.
-        if (ks != KS - 1) return;
+        if (ks != KS - 1 || (RBN == 1 && wave >= 4)) return;
         u32x4 got[TP][kMidFlaggedSlices - 1] = {};
         uint32_t *base = reinterpret_cast<uint32_t *>(partial) + wave * 256 + lane * 4;
         for (int spins = 0;; ++spins) {
@@ -623,6 +626,7 @@ __device__ __forceinline__ void mid_block(
     __syncthreads();
     if (!s_last) return;
     for (int item = wave; item < kItems; item += nw) {
+        if (RBN == 1 && (item & 4)) continue;
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int s2 = 0; s2 < KS; ++s2) {
             u32x4 v;
