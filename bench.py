@@ -40,7 +40,7 @@ TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median rep
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25781652, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25781838, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 
@@ -366,8 +366,8 @@ def main() -> int:
                     marlin_gemm.marlin_w4a16_gemm(x1[name], b, s, GROUP, out=o1[name])
                 marlin_gemm.marlin_w4a16_gemm(xs, sq[i % LAYERS][0], sq[i % LAYERS][1], GROUP, out=os_)
         elif args.profile in ("mid", "mid_m32"):
-            rows = 64 if args.profile == "mid" else 32   # 32: the mid-M kernel's one-row-block pass (gate+up at 32 rows
-            sweep = {"in_proj": (2560, 8192), "out_proj": (4096, 2560), **shapes}   # takes the two-slab small-M instance)
+            rows = 64 if args.profile == "mid" else 32   # 32: the mid-M kernel's one-row-block pass
+            sweep = {"in_proj": (2560, 8192), "out_proj": (4096, 2560), **shapes}
             sw = {name: [make_layer(*kn) for _ in range(8)] for name, kn in sweep.items() if name not in shapes}
             x64 = {name: torch.randn(rows, kn[0], device=dev).to(torch.bfloat16) for name, kn in sweep.items()}
             o64 = {name: torch.empty(rows, kn[1], dtype=torch.bfloat16, device=dev) for name, kn in sweep.items()}

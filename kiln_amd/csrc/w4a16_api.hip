@@ -478,10 +478,11 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // products of its 64-row pass), and with that it leads the two-slab small-M instance from the first row
 // beyond 16 on every shape (down projection at 17 / 32 rows 8.4 / 9.1 us against 9.7 / 12.5, out-projection
 // 6.4 / 6.7 against 7.8 / 8.4, in-projection 6.6 / 7.2 against 6.7 / 8.4, 4096 -> 14336 12.6 / 13.4 against
-// 15.3 / 21.2) but the wide outputs of a short K, which stay with the two-slab instance up to 32 rows
-// (gate+up 9.6 / 11.1 us against 10.8 / 11.2, 3584 -> 18944 17.6 / 18.9 against 21.6 / 22.1; with two groups
-// of A in flight in the one-row-block pass the kernel leads on 2560 -> 10240 and 12288 and 2048 -> 11008 from
-// some row between 24 and 32 on: 8.0 / 8.8 us against 8.1 / 8.3, so up to 12288 columns from 28).  With adapters 17
+// 15.3 / 21.2) but the wide outputs of a short K (K < 4096, N >= 10240), which stay with the two-slab instance up
+// to 20 rows: the mid-M kernel's time hardly grows with the rows of a run of up to 32 (gate+up 9.8 / 10.1 /
+// 10.4 us at 17 / 24 / 32 rows; all three pairs of a block meet in one phase there), the two-slab instance's
+// does (9.6 / 10.5 / 11.2), and they cross at 20...21 rows on gate+up, 2560 -> 10240 and 12288 and 2048 -> 11008
+// (3584 -> 18944: level, 19.2...19.6 us, at every row count).  With adapters 17
 // everywhere: the two-slab instance needs the projection from a launch in front, the mid-M kernel computes it
 // in its own first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.4 / 10.7 /
 // 13.4 / 13.7 us against 14.4 / 13.3 / 19.2 / 17.0).
@@ -490,11 +491,8 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // 2560 -> 12288 31.8 against 35.0, down projection at 192 rows 24.5 against 29.1 but 34.5 against 31.3 at 256);
 // up to 12 M: 320 rows (out-projection at 320 rows 16.1 against 23.1, 2560 -> 1024 8.7 against 16.2) -- while
 // on large ones it falls behind from 160 rows on (14336 -> 4096: 55 against 47 us; gate+up 42.5 against 35.2).
-constexpr int kMidMinM = 17, kMidMinMWideShortK = 33, kMidMinMWideShortKTo12288 = 28, kMidMaxM = 128, kMidMaxMSmallest = 320;
-int mid_min_rows(int n, int k, bool lora) {
-    if (lora || k >= 4096 || n < 10240) return kMidMinM;
-    return n <= 12288 ? kMidMinMWideShortKTo12288 : kMidMinMWideShortK;
-}
+constexpr int kMidMinM = 17, kMidMinMWideShortK = 21, kMidMaxM = 128, kMidMaxMSmallest = 320;
+int mid_min_rows(int n, int k, bool lora) { return !lora && k < 4096 && n >= 10240 ? kMidMinMWideShortK : kMidMinM; }
 int mid_max_rows(int n, int k) {
     const long long kn = (long long)k * n;
     if (kn <= 12ll << 20) return kMidMaxMSmallest;

@@ -473,11 +473,15 @@ __device__ __forceinline__ void mid_block(
     }
     KILN_MID_TL(5);  // main loop done
 
-    // --- the wavefronts' partial tiles meet in LDS, at most two pairs at a time (a wavefront's
-    // 16 KiB slot holds two pairs' tiles): every wavefront writes its own slot (item = (pair, row
-    // block, register quad q): rows 32 rb + 8 q + 4 h ... + 3 of column l32), then item i is summed
-    // over the wavefronts, in wavefront (= ascending K) order, by wavefront i % nw.
-    constexpr int kItems = TP * 2 * 4;
+    // --- the wavefronts' partial tiles meet in LDS, as many pairs at a time as a wavefront's 16 KiB slot
+    // holds (two with both row blocks, all of them with one): every wavefront writes its own slot (item =
+    // (pair, row block, register quad q): rows 32 rb + 8 q + 4 h ... + 3 of column l32; a pass over one row
+    // block has the items of that block only, packed), then every item is summed over the wavefronts, in
+    // wavefront (= ascending K) order, by one wavefront.
+    constexpr int kItems = TP * 2 * 4;         // ids of items: pair * 8 + row block * 4 + quad (as the partial tiles are laid out)
+    constexpr int kPerPair = RBN * 4;          // items of a pair in this pass, = their stride in a slot
+    constexpr int kPhasePairs = 16 / kPerPair; // pairs a slot holds
+    constexpr int kPhases = (TP + kPhasePairs - 1) / kPhasePairs;
     const int NT = N / kTileN;
     auto store_item = [&](f32x4 v, int item) {
         const int q = item & 3, rb = (item >> 2) & 1, p = item >> 3;
@@ -520,25 +524,25 @@ __device__ __forceinline__ void mid_block(
         return sum;
     };
     [[maybe_unused]] f32x4 own[TP];  // counter-free exchange, last slice: this wavefront's sums, one per pair
-    unrolled<0, (TP + 1) / 2>([&](auto phc) {
-        constexpr int p0 = 2 * decltype(phc)::value, p1 = p0 + 2 < TP ? p0 + 2 : TP;
+    unrolled<0, kPhases>([&](auto phc) {
+        constexpr int p0 = kPhasePairs * decltype(phc)::value, p1 = p0 + kPhasePairs < TP ? p0 + kPhasePairs : TP;
         if constexpr (p0 > 0) __syncthreads();  // the previous phase's sums have been read
 #pragma unroll
         for (int p = p0; p < p1; ++p)
 #pragma unroll
-            for (int rb = 0; rb < RBN; ++rb)  // (one row block per pass: nobody reads the other one's items below)
+            for (int rb = 0; rb < RBN; ++rb)
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
-                    mine[(((p - p0) * 2 + rb) * 4 + q) * 64 + lane] =
+                    mine[(((p - p0) * RBN + rb) * 4 + q) * 64 + lane] =
                         f32x4{acc[p][rb][4 * q], acc[p][rb][4 * q + 1], acc[p][rb][4 * q + 2], acc[p][rb][4 * q + 3]};
         __syncthreads();
         if constexpr (p0 == 0) KILN_MID_TL(6);  // every wavefront's tiles are in LDS
         if (flagged) {  // eight wavefronts: item (p0 + j) * 8 + wave for each pair j of the phase
-            if (RBN == 1 && wave >= 4) return;  // items of the row block this pass does not compute
+            if (wave >= kPerPair) return;  // (one row block per pass: four items a pair)
 #pragma unroll
             for (int j = 0; j < p1 - p0; ++j) {
                 const int item = (p0 + j) * 8 + wave;
-                const f32x4 sum = sum_over_wavefronts(item - p0 * 8);
+                const f32x4 sum = sum_over_wavefronts(j * kPerPair + wave);
                 if (ks == KS - 1) {
                     own[p0 + j] = sum;
                 } else {  // the complement of a sum's bits is never zero, so the part is its own arrival flag
@@ -549,9 +553,9 @@ __device__ __forceinline__ void mid_block(
             }
             return;
         }
-        for (int item = p0 * 8 + wave; item < p1 * 8; item += nw) {
-            if (RBN == 1 && (item & 4)) continue;  // an item of the row block this pass does not compute
-            const f32x4 sum = sum_over_wavefronts(item - p0 * 8);
+        for (int c = wave; c < (p1 - p0) * kPerPair; c += nw) {
+            const int item = (p0 + c / kPerPair) * 8 + c % kPerPair;
+            const f32x4 sum = sum_over_wavefronts(c);
             if (KS == 1) {
                 store_item(sum, item);
             } else {
@@ -570,7 +574,7 @@ __device__ __forceinline__ void mid_block(
         // it waits for is running or done.  Each part is loaded once per poll; the loads are
         // straight-line code up to their wait, so the parts of absent slices (zeros nobody
         // writes, or another run's parts) are loaded too and ignored.
-        if (ks != KS - 1 || (RBN == 1 && wave >= 4)) return;
+        if (ks != KS - 1 || wave >= kPerPair) return;
         u32x4 got[TP][kMidFlaggedSlices - 1] = {};
         uint32_t *base = reinterpret_cast<uint32_t *>(partial) + wave * 256 + lane * 4;
         for (int spins = 0;; ++spins) {
@@ -625,8 +629,8 @@ __device__ __forceinline__ void mid_block(
     }
     __syncthreads();
     if (!s_last) return;
-    for (int item = wave; item < kItems; item += nw) {
-        if (RBN == 1 && (item & 4)) continue;
+    for (int c = wave; c < TP * kPerPair; c += nw) {
+        const int item = (c / kPerPair) * 8 + c % kPerPair;
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int s2 = 0; s2 < KS; ++s2) {
             u32x4 v;
