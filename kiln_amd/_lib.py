@@ -83,7 +83,7 @@ TUNING_EXPORTS = (
     "kiln_w4a16_debug_prefill_bm", "kiln_w4a16_debug_prefill_nb_full", "kiln_w4a16_debug_decode_direct_max_m",
     "kiln_w4a16_debug_decode_group_major", "kiln_w4a16_debug_decode_runs_per_launch", "kiln_w4a16_debug_tune",
     "kiln_w4a16_debug_mid", "kiln_w4a16_debug_gmp", "kiln_w4a16_debug_flagged", "kiln_w4a16_debug_lora_fold",
-    "kiln_w4a16_debug_rowsum_fold",
+    "kiln_w4a16_debug_rowsum_fold", "kiln_w4a16_debug_mid_waves",
 )
 
 _libs: dict[bool, ctypes.CDLL] = {}
@@ -126,6 +126,7 @@ def use_shipped() -> None:
         L.kiln_w4a16_debug_flagged(-1)
         L.kiln_w4a16_debug_lora_fold(-1)
         L.kiln_w4a16_debug_rowsum_fold(-1)
+        L.kiln_w4a16_debug_mid_waves(0)
     _active_tuning = False
 
 

@@ -73,6 +73,7 @@ struct Tuning {
     int gmp_tiles = 0, gmp_waves = 0, gmp_ks = 0;   // > 0: the private-staging small-M instance with this plan
     int mid = -1;                     // 0 = never the mid-M kernel, 1 = wherever a plan fits (any row count), -1 = automatic
     int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
+    int mid_waves = 0;                // > 0: its wavefronts per block, at most
     int flagged = -1;                 // 0 = K slices always meet through counters, -1 = automatic
     int lora_fold = -1;               // 0 = the LoRA projection always runs as a launch of its own, -1 = automatic
     int rowsum_fold = -1;             // 0 = the matrix-core kernel's row sums always come from a launch in front, -1 = automatic
@@ -478,11 +479,12 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // products of its 64-row pass), and with that it leads the two-slab small-M instance from the first row
 // beyond 16 on every shape (down projection at 17 / 32 rows 8.4 / 9.1 us against 9.7 / 12.5, out-projection
 // 6.4 / 6.7 against 7.8 / 8.4, in-projection 6.6 / 7.2 against 6.7 / 8.4, 4096 -> 14336 12.6 / 13.4 against
-// 15.3 / 21.2) but the wide outputs of a short K (K < 4096, N >= 10240), which stay with the two-slab instance up
+// 15.3 / 21.2) but the wide outputs of a short K (K <= 3072, N >= 10240), which stay with the two-slab instance up
 // to 20 rows: the mid-M kernel's time hardly grows with the rows of a run of up to 32 (gate+up 9.8 / 10.1 /
 // 10.4 us at 17 / 24 / 32 rows; all three pairs of a block meet in one phase there), the two-slab instance's
 // does (9.6 / 10.5 / 11.2), and they cross at 20...21 rows on gate+up, 2560 -> 10240 and 12288 and 2048 -> 11008
-// (3584 -> 18944: level, 19.2...19.6 us, at every row count).  With adapters 17
+// (3584 -> 18944 was level, 19.2...19.6 us, until its 28 groups could go to ten wavefronts unsliced: 12.1 /
+// 13.1 us at 17 / 32 rows against 20.8 on the two-slab instance, hence the bound on K).  With adapters 17
 // everywhere: the two-slab instance needs the projection from a launch in front, the mid-M kernel computes it
 // in its own first blocks (two adapters at 24 rows, out- / in- / down- / gate+up projection: 10.4 / 10.7 /
 // 13.4 / 13.7 us against 14.4 / 13.3 / 19.2 / 17.0).
@@ -492,7 +494,7 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // up to 12 M: 320 rows (out-projection at 320 rows 16.1 against 23.1, 2560 -> 1024 8.7 against 16.2) -- while
 // on large ones it falls behind from 160 rows on (14336 -> 4096: 55 against 47 us; gate+up 42.5 against 35.2).
 constexpr int kMidMinM = 17, kMidMinMWideShortK = 21, kMidMaxM = 128, kMidMaxMSmallest = 320;
-int mid_min_rows(int n, int k, bool lora) { return !lora && k < 4096 && n >= 10240 ? kMidMinMWideShortK : kMidMinM; }
+int mid_min_rows(int n, int k, bool lora) { return !lora && k <= 3072 && n >= 10240 ? kMidMinMWideShortK : kMidMinM; }
 int mid_max_rows(int n, int k) {
     const long long kn = (long long)k * n;
     if (kn <= 12ll << 20) return kMidMaxMSmallest;
@@ -524,7 +526,7 @@ bool mid_flagged(const MidArgs &a) {
 // 40 rows, 4096 -> 11008 at 17: three pairs in two slices where two pairs unsliced would lead).  Eight
 // narrow outputs of a long K swept afterwards (4096 -> 512 ... 8192 -> 3072 at 24, 64 and 128 rows): within
 // 4 % of the best plan but on 6144 -> 1536 (6...12 %: 12 groups dealt to 8 wavefronts count as 16).
-MidPlan plan_mid(int m, int n, int k, int cus) {
+MidPlan plan_mid(int m, int n, int k, int cus, bool lora) {
     MidPlan best;
     const int G = k / kGroupK, runs = ceil_div(m, mid_max_rows_per_run());
     for (int pairs = 1; pairs <= 3; ++pairs) {
@@ -537,7 +539,14 @@ MidPlan plan_mid(int m, int n, int k, int cus) {
             a.K = k;
             a.KS = ks;
             a.GS = G / ks;
-            a.waves = a.GS < 8 ? a.GS : 8;
+            // Ten wavefronts where a launch may have them (up to 32 rows, no adapters) and eight
+            // would take four groups each or more: 5120 -> 13824 at 17...32 rows 16.7...17.3 us (eight cannot
+            // hold 40 groups: two slices) -> 13.0...13.9, 4096 -> 14336 12.0...12.4 -> 11.6...12.0.  Not below:
+            // 20 groups as 10 x 2 measured 2...9 % slower than as 4 x 3 + 4 x 2 (in-projection 6.4 -> 6.5 us,
+            // 2560 -> 2560 5.5 -> 5.85), the shorter main loop paid for by the start and the meeting of more wavefronts.
+            int max_waves = a.GS > 24 ? mid_max_waves(m, ks, lora) : 8;
+            if (g_tune.mid_waves > 0) max_waves = std::min(g_tune.mid_waves, mid_max_waves(m, ks, lora));
+            a.waves = a.GS < max_waves ? a.GS : max_waves;
             a.pairs = pairs;
             if (!mid_plan_ok(a)) continue;
             const int col_blocks = mid_column_blocks(a);
@@ -583,7 +592,7 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
          (!prefill_pinned && g_tune.prefill_min_m == 0 && m >= mid_min_rows(n, k, lora != 0) && m <= mid_max_rows(n, k)))) {
         // with adapters the projection runs in the launch's first blocks: plan for the chip less those
         const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
-        const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus);
+        const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus, lora != 0);
         if (mp.ok) {
             gp->mid = true;
             gp->mp = mp;
@@ -1121,6 +1130,7 @@ void kiln_w4a16_debug_mid(int mode, int pairs, int kslices) {
     g_tune.mid_pairs = pairs;
     g_tune.mid_ks = kslices;
 }
+void kiln_w4a16_debug_mid_waves(int waves) { g_tune.mid_waves = waves > 0 ? waves : 0; }
 void kiln_w4a16_debug_tune(int waves, int run, int kslices) {
     g_tune.force_waves = waves;
     g_tune.force_u = run;

@@ -60,6 +60,28 @@ def _mid_instances():
     return cases
 
 
+@pytest.mark.parametrize("m,k,n,forced", [
+    (32, 5120, 1024, 0), (17, 4096, 1280, 0), (24, 3584, 2560, 0),   # 40 / 32 / 28 groups: ten wavefronts by plan
+    (32, 2560, 2560, 10), (20, 2560, 8192, 10), (32, 1536, 768, 10),  # 20 and 12 groups: ten by override
+    (32, 5120, 1024, 8),                                              # and the same weights through eight (two K slices)
+    (32, 9216, 512, 0), (17, 18944, 256, 0),                          # K slices of 36 / 37 groups: ten, counter-free exchange
+])
+def test_ten_wavefronts_up_to_32_rows(oracle, m, k, n, forced):
+    """A launch of up to 32 rows may have ten wavefronts per block (ten slots of 16 KiB are all the LDS a
+    compute unit has); the planner takes them where eight would hold four groups of a slice each or more."""
+    L = _lib.load_tuning()
+    x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=k + n + forced)
+    b, s = pack.repack_gptq(q, s_bits, None, 128)
+    try:
+        L.kiln_w4a16_debug_mid(1, 1, {5120: 1 if forced != 8 else 0, 9216: 2, 18944: 4}.get(k, 1))
+        L.kiln_w4a16_debug_mid_waves(forced)
+        assert _takes_mid(L, m, n, k), (m, k, n)
+        _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
+    finally:
+        L.kiln_w4a16_debug_mid(-1, 0, 0)
+        L.kiln_w4a16_debug_mid_waves(0)
+
+
 @pytest.mark.parametrize("pairs,gs,ks", _mid_instances())
 def test_every_mid_instance(oracle, pairs, gs, ks):
     """Every (pairs of tiles per block, groups per wavefront) instance, with the groups dealt evenly

@@ -59,7 +59,7 @@ def test_sixteen_wavefronts_only_where_twelve_cannot_form_the_plan():
     # from: 17 rows; wide outputs of a short K stay with the two-slab small-M instance up to 20 rows
     (16, 9216, 2560, "small"), (17, 9216, 2560, "mid"), (17, 4096, 2560, "mid"), (17, 2560, 8192, "mid"),
     (17, 2560, 1024, "mid"), (24, 4096, 4096, "mid"), (32, 8192, 8192, "mid"), (32, 5120, 13824, "mid"),
-    (17, 2560, 18432, "small"), (20, 2560, 18432, "small"), (21, 2560, 18432, "mid"), (32, 3584, 18944, "mid"),
+    (17, 2560, 18432, "small"), (20, 2560, 18432, "small"), (21, 2560, 18432, "mid"), (17, 3584, 18944, "mid"),
     (20, 2560, 10240, "small"), (21, 2560, 10240, "mid"), (32, 2560, 12288, "mid"), (24, 2048, 11008, "mid"),
     # to: 128 rows; 192 / 256 / 320 on small weights
     (128, 2560, 18432, "mid"), (129, 2560, 18432, "matrix-core"), (160, 14336, 4096, "matrix-core"),
