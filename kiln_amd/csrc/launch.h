@@ -145,7 +145,7 @@ struct MidArgs {
     float lora_scales[8] = {};
 };
 bool mid_flagged_ok(const MidArgs &a);
-int mid_max_waves(int m, int ks, bool lora);  // wavefronts a block of such a launch may have
+int mid_max_waves(int m, int pairs, bool lora);  // wavefronts a block of such a launch may have
 int mid_column_blocks(const MidArgs &a);
 int mid_max_rows_per_run();
 bool mid_plan_ok(const MidArgs &a);

@@ -526,7 +526,7 @@ bool mid_flagged(const MidArgs &a) {
 // 40 rows, 4096 -> 11008 at 17: three pairs in two slices where two pairs unsliced would lead).  Eight
 // narrow outputs of a long K swept afterwards (4096 -> 512 ... 8192 -> 3072 at 24, 64 and 128 rows): within
 // 4 % of the best plan but on 6144 -> 1536 (6...12 %: 12 groups dealt to 8 wavefronts count as 16).
-MidPlan plan_mid(int m, int n, int k, int cus, bool lora) {
+MidPlan plan_mid_waves(int m, int n, int k, int cus, bool lora, bool ten_beyond_32_rows) {
     MidPlan best;
     const int G = k / kGroupK, runs = ceil_div(m, mid_max_rows_per_run());
     for (int pairs = 1; pairs <= 3; ++pairs) {
@@ -539,13 +539,17 @@ MidPlan plan_mid(int m, int n, int k, int cus, bool lora) {
             a.K = k;
             a.KS = ks;
             a.GS = G / ks;
-            // Ten wavefronts where a launch may have them (up to 32 rows, no adapters) and eight
+            // Ten wavefronts where a launch may have them (up to 32 rows, or one pair per block; no adapters) and eight
             // would take four groups each or more: 5120 -> 13824 at 17...32 rows 16.7...17.3 us (eight cannot
             // hold 40 groups: two slices) -> 13.0...13.9, 4096 -> 14336 12.0...12.4 -> 11.6...12.0.  Not below:
             // 20 groups as 10 x 2 measured 2...9 % slower than as 4 x 3 + 4 x 2 (in-projection 6.4 -> 6.5 us,
             // 2560 -> 2560 5.5 -> 5.85), the shorter main loop paid for by the start and the meeting of more wavefronts.
-            int max_waves = a.GS > 24 ? mid_max_waves(m, ks, lora) : 8;
-            if (g_tune.mid_waves > 0) max_waves = std::min(g_tune.mid_waves, mid_max_waves(m, ks, lora));
+            // Beyond 32 rows only blocks of one pair may have ten, and the 64-row pass with four groups to a
+            // wavefront waits for A more than this model knows (13824 -> 5120 at 64 rows 29.9 us in three slices
+            // of 10 x 4 against 26.0 in six of 8 x 3; 5120 -> 5120 15.2 against 13.1): there they are the plan of
+            // last resort (plan_mid).
+            int max_waves = a.GS > 24 && (m <= 32 || ten_beyond_32_rows) ? mid_max_waves(m, pairs, lora) : 8;
+            if (g_tune.mid_waves > 0) max_waves = std::min(g_tune.mid_waves, mid_max_waves(m, pairs, lora));
             a.waves = a.GS < max_waves ? a.GS : max_waves;
             a.pairs = pairs;
             if (!mid_plan_ok(a)) continue;
@@ -565,6 +569,15 @@ MidPlan plan_mid(int m, int n, int k, int cus, bool lora) {
         }
     }
     return best;
+}
+
+// The plan of eight wavefronts (ten up to 32 rows); where none exists -- 18944 = 148 groups = 4 x 37 -- and the
+// launch is one run of rows, one with ten wavefronts on blocks of one pair: 18944 -> 3584 at 48 / 64 rows 31 us
+// against 40.5 on the matrix-core kernel (at 128 rows 60 against 43: not beyond one run).
+MidPlan plan_mid(int m, int n, int k, int cus, bool lora) {
+    const MidPlan plan = plan_mid_waves(m, n, k, cus, lora, false);
+    if (plan.ok || m <= 32 || m > mid_max_rows_per_run()) return plan;
+    return plan_mid_waves(m, n, k, cus, lora, true);
 }
 
 MidArgs mid_args(const MidPlan &mp, int m, int n, int k) {

@@ -57,7 +57,7 @@ __device__ long long *g_mid_tl;
 #endif
 
 constexpr int kMidWaves = 8;                    // wavefronts per block, at most (and what the counter-free exchange takes)
-constexpr int kMidWavesOneRowBlock = 10;        // ... of a launch of up to 32 rows without adapters
+constexpr int kMidWavesMost = 10;               // ... of a launch of up to 32 rows, or of one pair per block, without adapters
 constexpr int kMidRows = 64;                    // rows per run
 constexpr int kMidSlotBytes = kMidRows * 256;   // one group of A: 64 rows x 128 bf16
 constexpr int kMidALoads = 16;                  // LDS-direct loads per group of A
@@ -652,11 +652,12 @@ __device__ __forceinline__ void mid_block(
 // at its own.
 constexpr int kMidOneRowBlock = 1, kMidTwoRowBlocks = 2, kMidRowBlocksByRun = 0;
 
-template <int ROW_BLOCKS>
-constexpr int kMidWavesOf = ROW_BLOCKS == kMidOneRowBlock ? kMidWavesOneRowBlock : kMidWaves;
+// (one pair per block: 114...153 registers whatever the row blocks, so ten wavefronts there too)
+template <int TP, int ROW_BLOCKS, bool LORA>
+constexpr int kMidWavesOf = !LORA && (ROW_BLOCKS == kMidOneRowBlock || TP == 1) ? kMidWavesMost : kMidWaves;
 
 template <int TP, int GPW, bool LORA, int ROW_BLOCKS>
-__global__ __launch_bounds__(kMidWavesOf<ROW_BLOCKS> * 64) void w4a16_mid_kernel(
+__global__ __launch_bounds__((kMidWavesOf<TP, ROW_BLOCKS, LORA> * 64)) void w4a16_mid_kernel(
     const uint16_t *__restrict__ A_all, const u32x4 *__restrict__ B, const uint16_t *__restrict__ S,
     uint16_t *__restrict__ C_all, float *partial_all, int *counters_all, int rows, int N, int K, int Gs, int KS,
     int GS, int full_waves, int swiglu, int flagged, int col_shift, MidLora lo) {
@@ -688,7 +689,7 @@ __global__ __launch_bounds__(kMidWavesOf<ROW_BLOCKS> * 64) void w4a16_mid_kernel
 
 template <int TP, int GPW, int ROW_BLOCKS>
 hipError_t launch_mid_tgs(const MidArgs &a, hipStream_t stream) {
-    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, ROW_BLOCKS>>(kMidWavesOf<ROW_BLOCKS> * kMidSlotBytes);
+    const hipError_t attr = allow_dynamic_lds<&w4a16_mid_kernel<TP, GPW, kMidLora, ROW_BLOCKS>>(kMidWavesOf<TP, ROW_BLOCKS, kMidLora> * kMidSlotBytes);
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
@@ -771,16 +772,17 @@ int mid_max_rows_per_run() { return kMidRows; }
 // What a launch of the mid-M kernel assumes: one to three pairs of tiles per block (N % 256 == 0
 // makes the tile count even; a last block may hold fewer pairs), equal K slices, at most eight
 // wavefronts of one to four groups each, every wavefront at least one group.
-// Up to 32 rows a group of A fills half a slot and a block's accumulators a third of the registers, so ten
-// wavefronts fit a compute unit's LDS (10 x 16 KiB) and registers; not with adapters (their blocks keep eight).
-int mid_max_waves(int m, int ks, bool lora) { return m <= 32 && !lora ? kMidWavesOneRowBlock : kMidWaves; }
+// Ten wavefronts fit a compute unit's LDS (10 x 16 KiB) and, three to a SIMD, hold at most 170 registers each:
+// the instances of a pass over one row block do (up to 32 rows), and those of one pair per block; not with
+// adapters (their blocks keep eight).
+int mid_max_waves(int m, int pairs, bool lora) { return !lora && (m <= 32 || pairs == 1) ? kMidWavesMost : kMidWaves; }
 
 bool mid_plan_ok(const MidArgs &a) {
     if (a.M < 1 || a.N < 256 || a.N % 256 != 0 || a.K < kGroupK || a.K % kGroupK != 0) return false;
     if (a.pairs < 1 || a.pairs > 3) return false;
     const int G = a.K / kGroupK;
     if (a.KS < 1 || a.GS < 1 || a.KS * a.GS != G) return false;
-    if (a.waves < 1 || a.waves > mid_max_waves(a.M, a.KS, a.r_total > 0) || a.waves > a.GS) return false;
+    if (a.waves < 1 || a.waves > mid_max_waves(a.M, a.pairs, a.r_total > 0) || a.waves > a.GS) return false;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     if (gpw > kMidMaxGroups || (a.pairs == 3 && gpw == 4)) return false;  // (3, 4) would spill registers
     const int full_waves = a.GS - a.waves * (gpw - 1);

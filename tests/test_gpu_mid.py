@@ -65,10 +65,12 @@ def _mid_instances():
     (32, 2560, 2560, 10), (20, 2560, 8192, 10), (32, 1536, 768, 10),  # 20 and 12 groups: ten by override
     (32, 5120, 1024, 8),                                              # and the same weights through eight (two K slices)
     (32, 9216, 512, 0), (17, 18944, 256, 0),                          # K slices of 36 / 37 groups: ten, counter-free exchange
+    (64, 18944, 512, 0), (48, 4736, 512, 0), (40, 4736, 512, 10),     # 37 groups a slice beyond 32 rows: no plan of eight
 ])
 def test_ten_wavefronts_up_to_32_rows(oracle, m, k, n, forced):
     """A launch of up to 32 rows may have ten wavefronts per block (ten slots of 16 KiB are all the LDS a
-    compute unit has); the planner takes them where eight would hold four groups of a slice each or more."""
+    compute unit has); the planner takes them where eight would hold four groups of a slice each or more.
+    Beyond 32 rows blocks of one pair may, where no plan of eight exists (37 groups a slice)."""
     L = _lib.load_tuning()
     x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=k + n + forced)
     b, s = pack.repack_gptq(q, s_bits, None, 128)
