@@ -403,10 +403,14 @@ SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n,
 // 16.2 us against 32.2 / 27.1 / 18.9 / 18.5) and behind from 96 rows on.  The one exception is the
 // widest projection at 49...64 rows, where one round of 64-row blocks (20.1 us) is ahead of two
 // runs (20.2...21.0).  Without such a plan the matrix-core kernel starts at 49 rows.
+int mid_max_rows(int n, int k);
 bool takes_prefill(int m, int n, int k, int cus) {
     if (g_tune.prefill_min_m > 0) return m >= g_tune.prefill_min_m;
     if (!slab_choice(32, n, k, cus, -1, -1, false).ok) return m >= 49;
     if ((long)n * k > (32L << 20) && m >= 49 && m <= 64) return true;
+    // rows beyond the one run the mid-M kernel takes on the largest weights of a long K: three passes of the
+    // small-M kernels over 64 MB and more of weights are behind one of the matrix-core kernel
+    if (m > mid_max_rows(n, k)) return true;
     return m >= 81;
 }
 
@@ -499,6 +503,11 @@ int mid_max_rows(int n, int k) {
     const long long kn = (long long)k * n;
     if (kn <= 12ll << 20) return kMidMaxMSmallest;
     if (kn <= 32ll << 20) return k <= 4096 ? 256 : 192;
+    // the largest weights with a long K: one run of rows (at 96 / 128 rows 8192 -> 8192 37.2 / 39.3 us against
+    // 37.2 / 36.3 on the matrix-core kernel, 5120 -> 13824 46.9 / 48.1 against 40.8 / 40.4, 13824 -> 5120 42.8 /
+    // 45.0 against 39.9 / 39.2, 18944 -> 3584 46.9 against 41.2 at 128; 3584 -> 18944, as large but of a short K,
+    // 39 / 40 against 50, and 14336 -> 4096, 56 M, level)
+    if (kn > 60ll << 20 && k >= 5120) return mid_max_rows_per_run();
     return kMidMaxM;
 }
 
@@ -532,13 +541,14 @@ MidPlan plan_mid_waves(int m, int n, int k, int cus, bool lora, bool ten_beyond_
     for (int pairs = 1; pairs <= 3; ++pairs) {
         if (g_tune.mid_pairs && pairs != g_tune.mid_pairs) continue;
         for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
-            if (G % ks != 0 || (g_tune.mid_ks && ks != g_tune.mid_ks)) continue;
+            // (a shorter last slice: not with adapters, nor in the plan of last resort below -- neither was measured)
+            if ((G % ks != 0 && (lora || ten_beyond_32_rows)) || (g_tune.mid_ks && ks != g_tune.mid_ks)) continue;
             MidArgs a{};
             a.M = m;
             a.N = n;
             a.K = k;
             a.KS = ks;
-            a.GS = G / ks;
+            a.GS = ceil_div(G, ks);  // the last slice may be shorter (mid_plan_ok says when)
             // Ten wavefronts where a launch may have them (up to 32 rows, or one pair per block; no adapters) and eight
             // would take four groups each or more: 5120 -> 13824 at 17...32 rows 16.7...17.3 us (eight cannot
             // hold 40 groups: two slices) -> 13.0...13.9, 4096 -> 14336 12.0...12.4 -> 11.6...12.0.  Not below:
@@ -557,7 +567,11 @@ MidPlan plan_mid_waves(int m, int n, int k, int cus, bool lora, bool ten_beyond_
             if ((size_t)runs * col_blocks * sizeof(int) > kCounterCapacity) continue;
             const int gpw = ceil_div(a.GS, a.waves), rounds = ceil_div(col_blocks * ks * runs, cus);
             const float exchange = ks == 1 ? 0.f : (mid_flagged(a) ? 0.5f * ks - 0.5f : 1.7f * ks - 1.9f);
-            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange + 2.0f * (rounds - 1);
+            // (a shorter last slice where even ones are clearly worse or do not exist: 13824 -> 5120 at 64 rows runs
+            // 26.6 us in six even slices and 28.4...30.1 in five of 22 + 22 + 22 + 22 + 20 groups, which this model
+            // would prefer by the 1.7 us of a slice's exchange)
+            const float uneven = G % ks != 0 ? 2.0f : 0.f;
+            const float cost = rounds * gpw * (0.75f + 0.55f * pairs) + 4.5f + exchange + 2.0f * (rounds - 1) + uneven;
             if (!best.ok || cost < best.cost) {
                 best.ok = true;
                 best.KS = ks;

@@ -202,9 +202,12 @@ __device__ __forceinline__ void mid_block(
     // are slow when they meet in one die's L2).
     const int cb = (bx + ks * col_shift) % ncb;
     const int tf = cb * (2 * TP);  // first 16-column tile of the block
-    // the first `full_waves` wavefronts own GPW groups each, the others GPW - 1
-    const bool full = wave < full_waves;
-    const int g_first = full ? wave * GPW : full_waves * GPW + (wave - full_waves) * (GPW - 1);
+    // the first `fw` wavefronts own GPW groups each, the others GPW - 1; the last slice may have fewer groups
+    // than the others (K in groups not a multiple of the slices) and then fewer wavefronts of GPW: its count
+    // rides in the argument's second byte
+    const int fw = (ks == KS - 1 ? full_waves >> 8 : full_waves) & 255;
+    const bool full = wave < fw;
+    const int g_first = full ? wave * GPW : fw * GPW + (wave - fw) * (GPW - 1);
     const int g0 = ks * GS + g_first;  // all slices have GS groups
     const int gs_mask = (Gs == 1) ? 0 : -1;
 
@@ -693,7 +696,8 @@ hipError_t launch_mid_tgs(const MidArgs &a, hipStream_t stream) {
     if (attr != hipSuccess) return attr;
     const int NT = a.N / kTileN;
     const int runs = (a.M + kMidRows - 1) / kMidRows;
-    const int full_waves = a.GS - a.waves * (GPW - 1);
+    const int last_groups = a.K / kGroupK - (a.KS - 1) * a.GS;  // of the last slice: GS, or fewer
+    const int full_waves = (a.GS - a.waves * (GPW - 1)) | ((last_groups - a.waves * (GPW - 1)) << 8);
     MidLora lo{};
     lo.t = (const uint16_t *)a.lora_t;
     lo.b = (const uint16_t *)a.lora_b;
@@ -781,12 +785,16 @@ bool mid_plan_ok(const MidArgs &a) {
     if (a.M < 1 || a.N < 256 || a.N % 256 != 0 || a.K < kGroupK || a.K % kGroupK != 0) return false;
     if (a.pairs < 1 || a.pairs > 3) return false;
     const int G = a.K / kGroupK;
-    if (a.KS < 1 || a.GS < 1 || a.KS * a.GS != G) return false;
+    // slices of GS groups; the last one may be shorter (11008 = 86 groups = 29 + 29 + 28), without adapters
+    if (a.KS < 1 || a.GS < 1 || a.KS * a.GS < G || (a.KS - 1) * a.GS >= G) return false;
+    if (a.KS * a.GS != G && a.r_total > 0) return false;
     if (a.waves < 1 || a.waves > mid_max_waves(a.M, a.pairs, a.r_total > 0) || a.waves > a.GS) return false;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     if (gpw > kMidMaxGroups || (a.pairs == 3 && gpw == 4)) return false;  // (3, 4) would spill registers
     const int full_waves = a.GS - a.waves * (gpw - 1);
-    return full_waves >= 1 && full_waves <= a.waves;
+    // the last slice: every wavefront gpw or gpw - 1 groups there too (none of gpw is fine)
+    const int last_full_waves = G - (a.KS - 1) * a.GS - a.waves * (gpw - 1);
+    return full_waves >= 1 && full_waves <= a.waves && last_full_waves >= 0 && last_full_waves <= a.waves;
 }
 
 // The counter-free exchange deals a pair's items (eight, or four of a pass over one row block) to the block's

@@ -84,6 +84,28 @@ def test_ten_wavefronts_up_to_32_rows(oracle, m, k, n, forced):
         L.kiln_w4a16_debug_mid_waves(0)
 
 
+@pytest.mark.parametrize("m,k,n,pairs,ks", [
+    (64, 11008, 512, 2, 4), (24, 11008, 512, 1, 3), (100, 11008, 768, 2, 3),   # 86 groups: 22 + 22 + 22 + 20, 29 + 29 + 28
+    (64, 18944, 256, 1, 7), (17, 8960, 512, 1, 3), (128, 2560, 512, 1, 3),      # 148 = 6 x 22 + 16; 70 = 24 + 24 + 22; 20 = 7 + 7 + 6
+    (40, 1408, 256, 1, 2), (32, 3200, 256, 1, 4),                               # 11 = 6 + 5 (a wavefront fewer); 25 = 7 + 7 + 7 + 4
+])
+def test_a_shorter_last_k_slice(oracle, m, k, n, pairs, ks):
+    """K in groups need not be a multiple of the slices: the last slice may have fewer groups (every wavefront
+    of it as many as in the other slices or one fewer).  Forced here; the planner takes such a plan where no
+    even slicing fits (11008 = 86 groups) or is clearly worse."""
+    L = _lib.load_tuning()
+    x, q, s_bits = oracle.gen_problem(m, k, n, 128, seed=k + n + ks)
+    b, s = pack.repack_gptq(q, s_bits, None, 128)
+    try:
+        L.kiln_w4a16_debug_mid(1, pairs, ks)
+        import ctypes
+        out = (ctypes.c_int * 8)()
+        assert L.kiln_w4a16_debug_gemm_plan(m, n, k, 256, out) == 0 and out[6] == 1 and out[7] == pairs * 16 + ks, list(out)
+        _run_case(oracle, m, k, n, 128, x, b, s, q, s_bits)
+    finally:
+        L.kiln_w4a16_debug_mid(-1, 0, 0)
+
+
 @pytest.mark.parametrize("pairs,gs,ks", _mid_instances())
 def test_every_mid_instance(oracle, pairs, gs, ks):
     """Every (pairs of tiles per block, groups per wavefront) instance, with the groups dealt evenly

@@ -64,6 +64,9 @@ def test_sixteen_wavefronts_only_where_twelve_cannot_form_the_plan():
     # to: 128 rows; 192 / 256 / 320 on small weights
     (128, 2560, 18432, "mid"), (129, 2560, 18432, "matrix-core"), (160, 14336, 4096, "matrix-core"),
     (64, 18944, 3584, "mid"), (65, 18944, 3584, "matrix-core"), (128, 18944, 3584, "matrix-core"),
+    # the largest weights with a long K: one run of rows; as large but of a short K: two
+    (64, 8192, 8192, "mid"), (65, 8192, 8192, "matrix-core"), (128, 5120, 13824, "matrix-core"), (128, 3584, 18944, "mid"),
+    (128, 14336, 4096, "mid"), (128, 11008, 4096, "mid"),
     (160, 8192, 8192, "matrix-core"),
     (192, 9216, 2560, "mid"), (193, 9216, 2560, "matrix-core"),
     (256, 2560, 8192, "mid"), (257, 2560, 8192, "matrix-core"), (256, 2560, 12288, "mid"),
@@ -76,9 +79,11 @@ def test_which_kernel_takes_a_row_count(m, k, n, want):
 @pytest.mark.parametrize("m,k,n,want", [
     (64, 2560, 8192, (1, 1)), (64, 4096, 2560, (1, 2)), (64, 2560, 18432, (3, 1)), (64, 9216, 2560, (1, 3)),
     # rounds after the first cost their start: no pile of short slices
-    (128, 5120, 13824, (3, 2)), (96, 3584, 18944, (2, 1)), (128, 3584, 18944, (2, 1)),
+    (64, 5120, 13824, (2, 2)), (96, 3584, 18944, (2, 1)), (128, 3584, 18944, (2, 1)),
     # ten wavefronts beyond 32 rows only where eight cannot form a plan (148 groups = 4 x 37), and in one run of rows
-    (64, 18944, 3584, (1, 4)), (64, 13824, 5120, (2, 6)), (64, 5120, 5120, (2, 2)),
+    (64, 13824, 5120, (2, 6)), (64, 5120, 5120, (2, 2)),
+    # a shorter last slice where K in groups has no even slicing that fits: 86 = 29 + 29 + 28, 148 = 6 x 22 + 16
+    (64, 11008, 4096, (2, 4)), (32, 11008, 4096, (2, 3)), (64, 18944, 3584, (2, 7)), (64, 8960, 1536, (1, 3)),
     # one round either way: four short slices through the counter-free exchange lead two long ones
     (64, 4096, 1024, (1, 4)), (17, 4096, 1024, (1, 4)), (128, 4096, 1024, (1, 4)),
 ])
