@@ -892,16 +892,18 @@ static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm, 
 // Relative cost of a plan in units of one 128-column block's group: whole rounds, then the
 // sliced round, then the exchange of its partial tiles (wider blocks take about 1.3 times as
 // long per group and exchange twice the data).
-// A 128-row block takes 1.5 times as long per group as a 64-row one, exchanges at twice the price per
-// slice, and its launch carries 8 units more (the row sums from a launch in front, a longer prologue and
+// A 128-row block takes 1.5 times as long per group as a 64-row one, exchanges at four times the price per
+// slice, and its launch carries 6 units more (the row sums from a launch in front, a longer prologue and
 // store): fitted to 98 cases -- 14 shapes at 400 ... 4096 rows, each with 64- and 128-row blocks forced --
-// on which the cheaper plan by this cost is the faster one or within 0.8 % of it on average (14 % at worst).
+// and to 72 more -- 12 shapes of other models at 129 ... 512 rows, the three block shapes forced -- on which
+// the cheaper plan by this cost is the faster one or within 0.8 % (the former) and 0.6 % (the latter) of it
+// on average, 18 % and 5 % at worst.
 static float plan_cost(int m, int n, int k, int cus, const PrefillPlan &p) {
     const int G = k / kGroupK, m_blocks = (m + p.bm - 1) / p.bm, n_blocks = n / p.bn;
     const float rows = p.bm == 128 ? 1.5f : 1.0f;
     const float per_group = (p.bn == 256 ? 1.3f : 1.0f) * rows;
-    const float per_slice = (p.bn == 256 ? (p.bm == 128 ? 2.0f : 1.0f) : 0.5f) * rows;
-    float cost = (float)((m_blocks * n_blocks) / cus) * G * per_group + (p.bm == 128 ? 8.f : 0.f);
+    const float per_slice = (p.bm == 128 ? 2.0f : 0.5f) * rows;
+    float cost = (float)((m_blocks * n_blocks) / cus) * G * per_group + (p.bm == 128 ? 6.f : 0.f);
     if (n_blocks > p.nb_full) {
         cost += (float)((G + p.ks - 1) / p.ks) * per_group;
         if (p.ks > 1) cost += per_slice * p.ks;
@@ -914,7 +916,9 @@ static float plan_cost(int m, int n, int k, int cus, const PrefillPlan &p) {
 // not by the matrix cores (rows past M are computed and dropped); 128 x 256 blocks (four wavefronts
 // side by side, each 128 x 64) where the chip is saturated: the best measured rate, because every
 // wavefront's weights are its own and A is shared by all four.  Which of the two, and which width
-// of the 64-row block: the lower modelled cost (plan_cost); up to 384 rows always 64.  (A fixed
+// of the 64-row block: the lower modelled cost (plan_cost); up to 128 rows always 64 (until the 129...512-row
+// sweep it was 384, and 128 x 256 blocks in K slices were missed where they lead by 15...25 %: 18944 -> 3584 at
+// 321 rows 81.5 us against 107, 28672 -> 8192 at 256 rows 150 against 173, 6144 -> 6144 at 321 rows 51 against 68).  (A fixed
 // switch at 768 rows was 5 % slower on average over the same 98 cases and 69 % at worst: narrow
 // outputs want 64 rows at any row count, large products 128 rows from 400 on.)
 // The 256-row shapes stay available through the overrides.
@@ -947,9 +951,13 @@ PrefillPlan plan_prefill(int m, int n, int k, int cus, int force_bn, int force_b
     PrefillPlan best = plan_for_shape(m, n, k, cus, force_bn == 128 ? 128 : 256, 64);
     if (force_bn != 128 && force_bn != 256) {
         const PrefillPlan narrow = plan_for_shape(m, n, k, cus, 128, 64);
-        if (plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, best)) best = narrow;
+        // (not as whole rounds plus a rest in five slices or more: 4096 -> 12288 at 129...192 rows ran 70.7 us as
+        // 85 whole column blocks and 11 in seven slices against 47.4 as 64 x 256 blocks, 6144 -> 6144 at 321 rows
+        // 103 against 68.5)
+        const bool rest_in_many_slices = narrow.nb_full > 0 && narrow.ks >= 5;
+        if (!rest_in_many_slices && plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, best)) best = narrow;
     }
-    if (m > 384 && force_bn != 128) {
+    if (m > 128 && force_bn != 128) {
         const PrefillPlan tall = plan_for_shape(m, n, k, cus, 256, 128, sliced_units);
         if (plan_cost(m, n, k, cus, tall) < plan_cost(m, n, k, cus, best)) best = tall;
     }

@@ -93,7 +93,9 @@ def test_mid_m_plans(m, k, n, want):
 
 @pytest.mark.parametrize("m,k,n,rows", [
     (2048, 2560, 18432, 128), (2048, 9216, 2560, 128), (4096, 2560, 18432, 128), (1024, 2560, 18432, 128),
-    (360, 2560, 18432, 64), (384, 9216, 2560, 64),                         # up to 384 rows always 64
+    (384, 9216, 2560, 64), (192, 2560, 18432, 64),
+    (321, 18944, 3584, 128), (256, 28672, 8192, 128), (321, 6144, 6144, 128),  # 128 x 256 in K slices from 129 rows where they lead
+    (192, 4096, 12288, 64), (192, 11008, 4096, 64),
     (1024, 2560, 1024, 64), (2048, 2560, 1024, 64), (4096, 2560, 1024, 64),  # narrow outputs at any row count
     (1024, 2560, 2048, 64),
     (512, 13824, 5120, 128), (512, 8192, 8192, 128), (768, 2560, 18432, 128),  # large products from 385 rows on
