@@ -403,7 +403,7 @@ SlabChoice slab_choice(int m, int n, int k, int cus, int thread_k, int thread_n,
 // 16.2 us against 32.2 / 27.1 / 18.9 / 18.5) and behind from 96 rows on.  The one exception is the
 // widest projection at 49...64 rows, where one round of 64-row blocks (20.1 us) is ahead of two
 // runs (20.2...21.0).  Without such a plan the matrix-core kernel starts at 49 rows.
-int mid_max_rows(int n, int k);
+int mid_max_rows(int n, int k, bool lora = false);
 bool takes_prefill(int m, int n, int k, int cus) {
     if (g_tune.prefill_min_m > 0) return m >= g_tune.prefill_min_m;
     if (!slab_choice(32, n, k, cus, -1, -1, false).ok) return m >= 49;
@@ -495,12 +495,22 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // To: 128 rows (two runs of 64); small weights keep it ahead of the matrix-core kernel's 64-row blocks for
 // longer -- K * N up to 32 M: 192 rows, 256 where K <= 4096 (in-projection at 256 rows 25.2 against 26.5 us,
 // 2560 -> 12288 31.8 against 35.0, down projection at 192 rows 24.5 against 29.1 but 34.5 against 31.3 at 256);
-// up to 12 M: 320 rows (out-projection at 320 rows 16.1 against 23.1, 2560 -> 1024 8.7 against 16.2) -- while
+// up to 12 M: 320 rows (out-projection at 320 rows 16.1 against 23.1, 2560 -> 1024 8.7 against 16.2), up to 9 M:
+// 512, up to 2.5 M: 1024 (mid_max_rows) -- while
 // on large ones it falls behind from 160 rows on (14336 -> 4096: 55 against 47 us; gate+up 42.5 against 35.2).
-constexpr int kMidMinM = 17, kMidMinMWideShortK = 21, kMidMaxM = 128, kMidMaxMSmallest = 320;
+constexpr int kMidMinM = 17, kMidMinMWideShortK = 21, kMidMaxM = 128, kMidMaxMSmallest = 320, kMidMaxMTiny = 512, kMidMaxMVerySmallest = 1024;
 int mid_min_rows(int n, int k, bool lora) { return !lora && k <= 3072 && n >= 10240 ? kMidMinMWideShortK : kMidMinM; }
-int mid_max_rows(int n, int k) {
+int mid_max_rows(int n, int k, bool lora) {
     const long long kn = (long long)k * n;
+    // the very smallest: to 1024 rows (1024 -> 1024 at 640...1024 rows 6.4...6.6 us against 13.4...14.6 on the
+    // matrix-core kernel, 1536 -> 1536 8.7...11.3 against 17...18.5, 2560 -> 1024 11.8...14.6 against 18.5...20; at 4 M
+    // 2048 -> 2048 and 4096 -> 1024 still lead by a sixth there but 1024 -> 4096 is behind from 640 on).
+    // Calls with adapters keep the 320 rows they were measured at.
+    if (kn <= 5ll << 19 && !lora) return kMidMaxMVerySmallest;
+    // the smallest weights: to 512 rows (at 448...512 rows 2560 -> 1024 9.2...9.4 us against 17.1...17.5 on the
+    // matrix-core kernel, 2048 -> 2048 9.8 against 18, 4096 -> 1024 12.3...12.7 against 22...23, 3072 -> 3072 17.2...17.8
+    // against 26; 4096 -> 2560, 10 M, is behind there: 29.7 against 26.2)
+    if (kn <= 9ll << 20 && !lora) return kMidMaxMTiny;
     if (kn <= 12ll << 20) return kMidMaxMSmallest;
     if (kn <= 32ll << 20) return k <= 4096 ? 256 : 192;
     // the largest weights with a long K: one run of rows (at 96 / 128 rows 8192 -> 8192 37.2 / 39.3 us against
@@ -616,7 +626,7 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
     const bool prefill_pinned = g_tune.prefill_bm != 0 || g_tune.prefill_bn != 0 || g_tune.prefill_ks != 0 || g_tune.prefill_nb_full >= 0;
     if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
         (g_tune.mid == 1 ||
-         (!prefill_pinned && g_tune.prefill_min_m == 0 && m >= mid_min_rows(n, k, lora != 0) && m <= mid_max_rows(n, k)))) {
+         (!prefill_pinned && g_tune.prefill_min_m == 0 && m >= mid_min_rows(n, k, lora != 0) && m <= mid_max_rows(n, k, lora != 0)))) {
         // with adapters the projection runs in the launch's first blocks: plan for the chip less those
         const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
         const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus, lora != 0);
@@ -746,10 +756,39 @@ struct LoraSpec {
 };
 
 // Bytes a call of m rows needs, made monotone in m: the largest need of any m' <= m.  The plan
-// (and with it the need) changes with m' only through the small-M and mid-M runs (m' <= 320 here; beyond
+// (and with it the need) changes with m' only through the small-M and mid-M runs (m' <= 1024 here; beyond
 // that only overrides keep a call on that path) and through the matrix-core kernel's row blocks
 // of 64 or 128 rows, so those m' are the ones evaluated.
+#ifndef KILN_W4A16_TUNING_HOOKS
+// What workspace_bytes_upto found, by its arguments: the sizing walks over hundreds of plans (0.35...0.55 ms
+// of host time from 512 rows on), and callers that size per call -- the Python wrappers do -- ask for the
+// same few shapes again and again.  Not in the tuning build, whose overrides change the answer.
+struct SizeKey {
+    int m, n, k, cus, thread_k, thread_n;
+    bool operator==(const SizeKey &o) const {
+        return m == o.m && n == o.n && k == o.k && cus == o.cus && thread_k == o.thread_k && thread_n == o.thread_n;
+    }
+};
+struct SizeKeyHash {
+    size_t operator()(const SizeKey &s) const {
+        size_t h = 1469598103934665603ull;
+        for (int v : {s.m, s.n, s.k, s.cus, s.thread_k, s.thread_n}) h = (h ^ (size_t)(unsigned)v) * 1099511628211ull;
+        return h;
+    }
+};
+std::mutex g_size_mutex;
+std::unordered_map<SizeKey, size_t, SizeKeyHash> g_size_cache;
+#endif
+
 size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thread_n) {
+#ifndef KILN_W4A16_TUNING_HOOKS
+    const SizeKey key{m, n, k, cus, thread_k, thread_n};
+    {
+        std::lock_guard<std::mutex> lock(g_size_mutex);
+        auto it = g_size_cache.find(key);
+        if (it != g_size_cache.end()) return it->second;
+    }
+#endif
     size_t most = 0;
     auto consider = [&](int mm) {
         for (int lora = 0; lora < 3; ++lora) {  // a call with adapters may take another path
@@ -759,10 +798,15 @@ size_t workspace_bytes_upto(int m, int n, int k, int cus, int thread_k, int thre
             if (need > most) most = need;
         }
     };
-    const int small = g_tune.prefill_min_m > kMidMaxMSmallest ? g_tune.prefill_min_m : kMidMaxMSmallest;
+    const int small = g_tune.prefill_min_m > kMidMaxMVerySmallest ? g_tune.prefill_min_m : kMidMaxMVerySmallest;
     for (int mm = 1; mm <= m && mm <= small; ++mm) consider(mm);
     for (int mm = 64; mm < m; mm += 64) consider(mm);
     consider(m);
+#ifndef KILN_W4A16_TUNING_HOOKS
+    std::lock_guard<std::mutex> lock(g_size_mutex);
+    if (g_size_cache.size() > 4096) g_size_cache.clear();  // a caller cycling through many shapes
+    g_size_cache.emplace(key, most);
+#endif
     return most;
 }
 

@@ -955,7 +955,13 @@ PrefillPlan plan_prefill(int m, int n, int k, int cus, int force_bn, int force_b
         // 85 whole column blocks and 11 in seven slices against 47.4 as 64 x 256 blocks, 6144 -> 6144 at 321 rows
         // 103 against 68.5)
         const bool rest_in_many_slices = narrow.nb_full > 0 && narrow.ks >= 5;
-        if (!rest_in_many_slices && plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, best)) best = narrow;
+        // Two wavefronts a block: for outputs too narrow to give the wider block enough tiles (2560 -> 1024 at
+        // 400...4096 rows 17...36 us against 27...43).  On wider outputs the model's 1.0 : 1.3 a group does not hold
+        // where a compute unit gets one such block (3584 -> 4608 at 448 rows, 252 tiles: 65 us, 38...44 in the other
+        // shapes), and over 170 forced cases it never led by more than 3 % there.
+        const bool narrow_output = n <= 2048;
+        if (narrow_output && !rest_in_many_slices && plan_cost(m, n, k, cus, narrow) <= plan_cost(m, n, k, cus, best))
+            best = narrow;
     }
     if (m > 128 && force_bn != 128) {
         const PrefillPlan tall = plan_for_shape(m, n, k, cus, 256, 128, sliced_units);

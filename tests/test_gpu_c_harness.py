@@ -52,7 +52,7 @@ def test_golden_vectors_through_the_cpp_harness(tmp_path, tag, m, k, n, g):
     (16, 9216, 2560, 128),    # three K slices meeting in the zero-kept region
     (16, 2560, 18432, 128),   # the headline launch
     (64, 4096, 2560, 128),    # mid-M kernel, K sliced
-    (400, 2560, 2560, -1),    # matrix-core kernel, K sliced, one scale per column
+    (600, 2560, 2560, -1),    # matrix-core kernel, K sliced, one scale per column
 ])
 def test_four_host_threads_enter_the_library_at_once(oracle, tmp_path, m, k, n, g):
     """Own stream, workspace and output per thread, first calls racing on a plan cache that has never

@@ -22,7 +22,7 @@ CASES = [
     (600, 2560, 12288, True),    # 128-row blocks below 768 rows
     (2500, 4096, 2560, True),    # the most producers a launch takes
     (2048, 2560, 18432, False),  # several rounds of blocks: the launch in front stays
-    (400, 2560, 2560, False),    # the blocks sum their rows themselves
+    (400, 4096, 2560, False),    # the blocks sum their rows themselves
 ]
 IN_FRONT, OWN_ROWS, OTHER_KERNEL = 0, -2, -3
 
@@ -39,7 +39,7 @@ def test_the_plan_query_says_where_the_row_sums_come_from():
         if inside:
             assert p % 8 == 0 and 8 <= p <= 128 and p >= (m + 63) // 64
     assert L.kiln_w4a16_debug_prefill_rowsum_producers(2048, 18432, 2560, _cus()) == IN_FRONT
-    assert L.kiln_w4a16_debug_prefill_rowsum_producers(400, 2560, 2560, _cus()) == OWN_ROWS
+    assert L.kiln_w4a16_debug_prefill_rowsum_producers(400, 2560, 4096, _cus()) == OWN_ROWS
     assert L.kiln_w4a16_debug_prefill_rowsum_producers(16, 2560, 2560, _cus()) == OTHER_KERNEL
     try:
         L.kiln_w4a16_debug_rowsum_fold(0)

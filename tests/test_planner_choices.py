@@ -71,6 +71,8 @@ def test_sixteen_wavefronts_only_where_twelve_cannot_form_the_plan():
     (192, 9216, 2560, "mid"), (193, 9216, 2560, "matrix-core"),
     (256, 2560, 8192, "mid"), (257, 2560, 8192, "matrix-core"), (256, 2560, 12288, "mid"),
     (320, 4096, 2560, "mid"), (321, 4096, 2560, "matrix-core"), (320, 2560, 1024, "mid"),
+    (1024, 2560, 1024, "mid"), (1025, 2560, 1024, "matrix-core"), (512, 3072, 3072, "mid"), (448, 2048, 2048, "mid"),
+    (513, 2048, 2048, "matrix-core"), (1024, 1536, 1536, "mid"),
 ])
 def test_which_kernel_takes_a_row_count(m, k, n, want):
     assert _route(m, k, n)[0] == want
@@ -96,7 +98,8 @@ def test_mid_m_plans(m, k, n, want):
     (384, 9216, 2560, 64), (192, 2560, 18432, 64),
     (321, 18944, 3584, 128), (256, 28672, 8192, 128), (321, 6144, 6144, 128),  # 128 x 256 in K slices from 129 rows where they lead
     (192, 4096, 12288, 64), (192, 11008, 4096, 64),
-    (1024, 2560, 1024, 64), (2048, 2560, 1024, 64), (4096, 2560, 1024, 64),  # narrow outputs at any row count
+    (448, 3584, 4608, 128),                                                # (was 64 x 128, one block of two wavefronts a unit: 65 us)
+    (1025, 2560, 1024, 64), (2048, 2560, 1024, 64), (4096, 2560, 1024, 64),  # narrow outputs at any row count
     (1024, 2560, 2048, 64),
     (512, 13824, 5120, 128), (512, 8192, 8192, 128), (768, 2560, 18432, 128),  # large products from 385 rows on
     (512, 9216, 2560, 64), (512, 2560, 8192, 64),
