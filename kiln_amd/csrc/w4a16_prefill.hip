@@ -931,9 +931,13 @@ PrefillPlan plan_prefill(int m, int n, int k, int cus, int force_bn, int force_b
     int sliced_units = 0;
     {
         const int tiles = ((m + 127) / 128) * (n / 256);
-        if (2 * tiles > cus && tiles < cus) {
+        if (2 * tiles >= cus && tiles < cus) {
             const int ks = 2 * cus / tiles;
-            if (ks >= 2 && k / kGroupK / ks >= 24) sliced_units = 2 * cus;
+            // (shorter slices where the tiles leave a quarter of the units idle or more: 160 tiles of 8192 -> 10240 at
+            // 448...512 rows in three slices of 21 / 22 groups 103.5 us against 119 in two and 114...125 in 64-row
+            // blocks; 128 tiles of 8192 -> 8192, 14336 -> 8192, 28672 -> 8192 in four slices 3...8 % ahead of two)
+            const int min_groups = 4 * tiles <= 3 * cus ? 16 : 24;
+            if (ks >= 2 && k / kGroupK / ks >= min_groups) sliced_units = 2 * cus;
         }
     }
     if (force_bm == 64 || force_bm == 128 || force_bm == 256) {
