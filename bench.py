@@ -40,7 +40,7 @@ TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median rep
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25781604, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25781555, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 
