@@ -84,6 +84,15 @@ def test_ten_wavefronts_up_to_32_rows(oracle, m, k, n, forced):
         L.kiln_w4a16_debug_mid_waves(0)
 
 
+def test_new_plans_with_one_scale_per_column(oracle):
+    """groupsize = -1 through ten wavefronts, a shorter last slice, and 1000 rows on a small weight."""
+    for m, k, n in ((32, 5120, 512), (64, 11008, 512), (1000, 1024, 1024)):
+        assert _takes_mid(_lib.load(), m, n, k), (m, k, n)
+        x, q, s_bits = oracle.gen_problem(m, k, n, -1, seed=m + k)
+        b, s = pack.repack_gptq(q, s_bits, None, -1)
+        _run_case(oracle, m, k, n, -1, x, b, s, q, s_bits)
+
+
 @pytest.mark.parametrize("m,k,n,pairs,ks", [
     (64, 11008, 512, 2, 4), (24, 11008, 512, 1, 3), (100, 11008, 768, 2, 3),   # 86 groups: 22 + 22 + 22 + 20, 29 + 29 + 28
     (64, 18944, 256, 1, 7), (17, 8960, 512, 1, 3), (128, 2560, 512, 1, 3),      # 148 = 6 x 22 + 16; 70 = 24 + 24 + 22; 20 = 7 + 7 + 6

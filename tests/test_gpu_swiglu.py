@@ -34,6 +34,9 @@ def _problem(oracle, m, k, n_out, g, seed, sigma=1.0):
     (16, 2560, 9216, 128, 1.0), (24, 2560, 9216, 128, 1.0), (40, 9216, 1280, 128, 1.0),
     (33, 2560, 1024, 128, 1.0), (64, 2560, 9216, 128, 1.0), (100, 512, 256, 128, 1.0), (128, 2560, 9216, 128, 1.0),
     (300, 2560, 2560, 128, 0.5), (1000, 1024, 4096, 128, 0.5), (2048, 2560, 9216, 128, 0.5),
+    # plans of the mid-M kernel that other models' shapes take: ten wavefronts (40 groups unsliced, up to 32 rows), a
+    # shorter last K slice (86 groups), both with the fused store; and its longer row range on small weights
+    (32, 5120, 512, 128, 1.0), (48, 11008, 512, 128, 1.0), (24, 11008, 256, 128, 1.0), (700, 1024, 512, 128, 0.5),
 ])
 def test_swiglu_cases(oracle, m, k, n_out, g, sigma):
     x, b_gu, s_gu, h_ref = _problem(oracle, m, k, n_out, g, seed=m + k + n_out, sigma=sigma)
