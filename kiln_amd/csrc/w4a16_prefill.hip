@@ -907,6 +907,13 @@ static float plan_cost(int m, int n, int k, int cus, const PrefillPlan &p) {
     if (n_blocks > p.nb_full) {
         cost += (float)((G + p.ks - 1) / p.ks) * per_group;
         if (p.ks > 1) cost += per_slice * p.ks;
+        // 128-row blocks sit two to a unit: behind whole rounds, the blocks of a K-sliced rest run beside the last round's
+        // and hold it up by their own length, in proportion to how many of them there are (gate+up at 640
+        // rows, 255 whole tiles and 105 in two slices of ten groups: 87.5 us, 73 with every tile whole or in
+        // 64-row blocks; at 512 rows, 32 tiles in five slices of four groups: nothing)
+        // (0.75 of that, and nothing for a rest of whole tiles, which is a round like the others: fitted with the rest)
+        if (p.bm == 128 && p.nb_full > 0 && p.ks > 1)
+            cost += 0.75f * (float)((n_blocks - p.nb_full) * m_blocks * p.ks) / cus * ((G + p.ks - 1) / p.ks) * per_group;
     }
     return cost;
 }
