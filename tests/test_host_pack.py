@@ -431,6 +431,20 @@ def test_workspace_bytes_is_monotone_in_m(k, n):
     assert tuned[15] >= sizes[15] or tuned[15] >= L.kiln_w4a16_workspace_zeroed_bytes()
 
 
+def test_memoised_workspace_sizes_equal_the_computed_ones():
+    """The shipped library remembers the size it computed for (m, n, k, overrides); the tuning build computes it
+    every time.  Both must agree, on first and on repeated queries, also where the mid-M kernel's row range ends."""
+    shipped, tuning = _lib.load(), ctypes.CDLL(str(_lib.TUNING_LIB_PATH))
+    for f in (tuning.kiln_w4a16_workspace_bytes, tuning.kiln_w4a16_workspace_bytes_tuned):
+        f.restype = ctypes.c_size_t
+    for k, n in MODEL_SHAPES + [(11008, 4096), (1024, 1024), (2560, 1024), (18944, 3584)]:
+        for m in (1, 16, 17, 64, 65, 128, 320, 512, 1024, 1025, 4096):
+            want = tuning.kiln_w4a16_workspace_bytes(m, n, k)
+            assert shipped.kiln_w4a16_workspace_bytes(m, n, k) == want, (m, k, n)
+            assert shipped.kiln_w4a16_workspace_bytes(m, n, k) == want, (m, k, n)
+            assert shipped.kiln_w4a16_workspace_bytes_tuned(m, n, k, 128, 16, -1) == tuning.kiln_w4a16_workspace_bytes_tuned(m, n, k, 128, 16, -1)
+
+
 def test_workspace_is_small_where_nothing_is_exchanged():
     """Decode calls need little more than the zeroed prefix -- the counters and the region in which
     K slices exchange their parts without counters, which is where the down projection's three
