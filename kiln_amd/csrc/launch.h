@@ -145,6 +145,7 @@ struct MidArgs {
     float lora_scales[8] = {};
 };
 bool mid_flagged_ok(const MidArgs &a);
+bool mid_lora_fold_ok(const MidArgs &a);  // the projection onto the adapters inside the launch: do its fields allow it?
 int mid_max_waves(int m, int pairs, bool lora);  // wavefronts a block of such a launch may have
 int mid_column_blocks(const MidArgs &a);
 int mid_max_rows_per_run();

@@ -885,20 +885,23 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             int kz = lora_project_slices(prob_m, prob_k);
             const int per_slice = ((steps + kz - 1) / kz + 3) / 4 * 4;  // whole 128-value groups
             kz = (steps + per_slice - 1) / per_slice;
-            if (g_tune.lora_fold != 0 && ma.waves >= 4 && lora->n_adapters <= 8) {
-                ma.lora_slices = kz;
-                ma.lora_producers = row_tiles * kz;
-                ma.lora_steps_per_slice = per_slice;
-                ma.lora_a = lora->a;
-                ma.lora_words = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
-                ma.lora_adapters = lora->n_adapters;
+            MidArgs folded = ma;
+            folded.lora_slices = kz;
+            folded.lora_producers = row_tiles * kz;
+            folded.lora_steps_per_slice = per_slice;
+            folded.lora_a = lora->a;
+            folded.lora_words = reinterpret_cast<unsigned *>(ws + kFoldFlagOffset);
+            folded.lora_adapters = lora->n_adapters;
+            // (what the launch itself checks: beyond four runs of rows, or more (slice, tile) words than a copy
+            // holds, the projection runs in front -- a call of 320 rows with adapters was refused here once)
+            if (g_tune.lora_fold != 0 && lora->n_adapters <= 8 && mid_lora_fold_ok(folded)) {
                 int end = 0;
                 for (int i = 0; i < 8; ++i) {
                     if (i < lora->n_adapters) end += lora->ranks[i];
-                    ma.lora_ends[i] = end;
-                    ma.lora_scales[i] = i < lora->n_adapters ? lora->scales[i] : 0.f;
+                    folded.lora_ends[i] = end;
+                    folded.lora_scales[i] = i < lora->n_adapters ? lora->scales[i] : 0.f;
                 }
-                return launch_mid(ma, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
+                return launch_mid(folded, st) == hipSuccess ? KILN_W4A16_OK : KILN_W4A16_ERR_LAUNCH;
             }
             PrefillArgs pj{};
             pj.A = A;

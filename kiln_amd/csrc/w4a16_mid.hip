@@ -754,15 +754,7 @@ hipError_t launch_mid_t(const MidArgs &a, int gpw, hipStream_t stream) {
 hipError_t launch_mid_lora(const MidArgs &a, hipStream_t stream) {
     if (a.r_total < 8 || a.r_total > 64 || a.r_total % 8 != 0 || !a.lora_t || !a.lora_b || a.lora_slices < 1)
         return hipErrorInvalidValue;
-    if (a.lora_producers > 0) {
-        // the projection's blocks: 256 working threads, 16-row tiles, words for (slice, tile) in a copy's 4 KiB
-        const int row_tiles = (a.M + 15) / 16;
-        if (a.waves < 4 || a.lora_slices > 16 || row_tiles * a.lora_slices > kLoraFoldReplicaWords - kMidFoldTileWord ||
-            a.lora_producers != row_tiles * a.lora_slices || !a.lora_a || !a.lora_words || a.lora_adapters < 1 ||
-            a.lora_adapters > 8 || a.lora_steps_per_slice < 4 || a.lora_steps_per_slice % 4 != 0 ||
-            (long)a.lora_slices * a.lora_steps_per_slice * 32 < a.K || a.M > 4 * kMidRows)
-            return hipErrorInvalidValue;
-    }
+    if (a.lora_producers > 0 && !mid_lora_fold_ok(a)) return hipErrorInvalidValue;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     switch (a.pairs) {
         case 1: return launch_mid_t<1>(a, gpw, stream);
@@ -772,6 +764,17 @@ hipError_t launch_mid_lora(const MidArgs &a, hipStream_t stream) {
 }
 #else
 int mid_max_rows_per_run() { return kMidRows; }
+
+// May the projection onto the adapters run in this launch's first blocks?  Those blocks: 256 working threads,
+// 16-row tiles, words for (slice, tile) in a copy's 4 KiB; up to four runs of rows.
+bool mid_lora_fold_ok(const MidArgs &a) {
+    const int row_tiles = (a.M + 15) / 16;
+    return a.waves >= 4 && a.lora_slices >= 1 && a.lora_slices <= 16 &&
+           row_tiles * a.lora_slices <= kLoraFoldReplicaWords - kMidFoldTileWord &&
+           a.lora_producers == row_tiles * a.lora_slices && a.lora_a && a.lora_words && a.lora_adapters >= 1 &&
+           a.lora_adapters <= 8 && a.lora_steps_per_slice >= 4 && a.lora_steps_per_slice % 4 == 0 &&
+           (long)a.lora_slices * a.lora_steps_per_slice * 32 >= a.K && a.M <= 4 * kMidRows;
+}
 
 // What a launch of the mid-M kernel assumes: one to three pairs of tiles per block (N % 256 == 0
 // makes the tile count even; a last block may hold fewer pairs), equal K slices, at most eight

@@ -51,6 +51,17 @@ def test_lora_on_few_rows(oracle, m, k, n):
     _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=3 * m + n, sigma_ab=0.05)
 
 
+@pytest.mark.parametrize("m,k,n", [
+    (192, 2560, 8192), (256, 4096, 2560), (257, 4096, 2560), (300, 2560, 2560), (320, 4096, 2560), (320, 2560, 1024),
+    (321, 2560, 1024),
+])
+def test_lora_where_small_weights_keep_the_mid_m_kernel(oracle, m, k, n):
+    """Small weights keep the mid-M kernel up to 192 ... 320 rows with adapters.  Up to four runs of rows
+    (256) the projection runs in the launch's first blocks, beyond that in a launch in front (a call of 320
+    rows was once refused: the dispatcher asked for the former where the launch only takes the latter)."""
+    _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=5 * m + n, sigma_ab=0.05)
+
+
 @pytest.mark.parametrize("mode", [0, 1, 2])
 @pytest.mark.parametrize("m,k,n,ranks", [
     (16, 2560, 4096, (16, 32)),
