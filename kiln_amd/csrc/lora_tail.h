@@ -113,7 +113,7 @@ struct LoraFold {
 };
 constexpr int kLoraFoldMaxProducers = 16;
 constexpr int kLoraFoldMaxAdapters = 4;
-constexpr int kLoraFoldStepsPerWave = 8;   // 32-value steps of K one producer wavefront takes, at most
+constexpr int kLoraFoldStepsPerWave = 12;  // 32-value steps of K one producer wavefront takes, at most
 constexpr int kLoraFoldReplicas = 16;
 constexpr int kLoraFoldReplicaWords = 1024;                  // 4 KiB from one replica to the next
 constexpr int kLoraFoldCountWord = kLoraFoldMaxProducers;    // a replica's reader count

@@ -75,7 +75,8 @@ struct Tuning {
     int mid_pairs = 0, mid_ks = 0;    // its tile pairs per block and K slices
     int mid_waves = 0;                // > 0: its wavefronts per block, at most
     int flagged = -1;                 // 0 = K slices always meet through counters, -1 = automatic
-    int lora_fold = -1;               // 0 = the LoRA projection always runs as a launch of its own, -1 = automatic
+    int lora_fold = -1;               // 0 = the LoRA projection always runs as a launch of its own, -1 = automatic,
+                                      // 2 = in the launch wherever the kernel can (whatever the grid's size)
     int rowsum_fold = -1;             // 0 = the matrix-core kernel's row sums always come from a launch in front, -1 = automatic
 };
 #ifdef KILN_W4A16_TUNING_HOOKS
@@ -551,8 +552,8 @@ MidPlan plan_mid_waves(int m, int n, int k, int cus, bool lora, bool ten_beyond_
     for (int pairs = 1; pairs <= 3; ++pairs) {
         if (g_tune.mid_pairs && pairs != g_tune.mid_pairs) continue;
         for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
-            // (a shorter last slice: not with adapters, nor in the plan of last resort below -- neither was measured)
-            if ((G % ks != 0 && (lora || ten_beyond_32_rows)) || (g_tune.mid_ks && ks != g_tune.mid_ks)) continue;
+            // (a shorter last slice: not in the plan of last resort below, which was not measured with one)
+            if ((G % ks != 0 && ten_beyond_32_rows) || (g_tune.mid_ks && ks != g_tune.mid_ks)) continue;
             MidArgs a{};
             a.M = m;
             a.N = n;
@@ -945,9 +946,11 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
         fold_probe.lora_steps_per_slice = fold_steps;
         fold_probe.lora_rows = prob_m;
         fold_probe.lora_adapters = lora->n_adapters;
-        // the producers take compute units of their own: only where the launch still fits the chip in one
-        // round (the in-projection's 256 blocks do not: 12.6 us folded against 10.6 with the launch of its own)
-        fold = decode_gmp_fold_ok(fold_probe) && gp.dl[0].plan.BPS * gp.dl[0].plan.KS + kz <= cus;
+        // the producers take compute units of their own: where the launch still fits the chip in one round
+        // (the in-projection's 256 blocks do not: 12.6 us folded against 10.6 with the launch of its own), or
+        // runs in several rounds anyway (5120 -> 13824, 432 blocks: 14.8 us folded against 18.8)
+        const int blocks = gp.dl[0].plan.BPS * gp.dl[0].plan.KS;
+        fold = decode_gmp_fold_ok(fold_probe) && (blocks + kz <= cus || blocks > cus || g_tune.lora_fold == 2);
         if (fold) {
             lora_slices = kz;
             rp = (lora->r_total + 15) / 16 * 16;

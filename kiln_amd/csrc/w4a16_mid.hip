@@ -788,9 +788,8 @@ bool mid_plan_ok(const MidArgs &a) {
     if (a.M < 1 || a.N < 256 || a.N % 256 != 0 || a.K < kGroupK || a.K % kGroupK != 0) return false;
     if (a.pairs < 1 || a.pairs > 3) return false;
     const int G = a.K / kGroupK;
-    // slices of GS groups; the last one may be shorter (11008 = 86 groups = 29 + 29 + 28), without adapters
+    // slices of GS groups; the last one may be shorter (11008 = 86 groups = 29 + 29 + 28)
     if (a.KS < 1 || a.GS < 1 || a.KS * a.GS < G || (a.KS - 1) * a.GS >= G) return false;
-    if (a.KS * a.GS != G && a.r_total > 0) return false;
     if (a.waves < 1 || a.waves > mid_max_waves(a.M, a.pairs, a.r_total > 0) || a.waves > a.GS) return false;
     const int gpw = (a.GS + a.waves - 1) / a.waves;
     if (gpw > kMidMaxGroups || (a.pairs == 3 && gpw == 4)) return false;  // (3, 4) would spill registers

@@ -52,6 +52,27 @@ def test_lora_on_few_rows(oracle, m, k, n):
 
 
 @pytest.mark.parametrize("m,k,n", [
+    (1, 18944, 3584), (16, 18944, 3584),   # the projection's wavefronts take ten steps of K each
+    (5, 5120, 13824), (16, 5120, 13824),   # a launch of more blocks than compute units, the projection in its first ones
+    (16, 11008, 4096),                     # as many blocks as compute units: the projection runs in front
+])
+def test_lora_on_few_rows_of_other_models_weights(oracle, m, k, n):
+    _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=5 * m + n, sigma_ab=0.05)
+
+
+@pytest.mark.parametrize("m", [17, 32, 48, 64, 100, 128])
+@pytest.mark.parametrize("k,n", [(11008, 512), (8960, 256)])
+def test_lora_with_a_shorter_last_k_slice(oracle, m, k, n):
+    """86 and 70 groups of K have no even slicing that fits the mid-M kernel's wavefronts: its last slice is
+    shorter, with adapters as without."""
+    import ctypes
+    from kiln_amd import _lib
+    out = (ctypes.c_int * 8)()
+    assert _lib.load().kiln_w4a16_debug_gemm_plan(m, n, k, 256, out) == 0 and out[6] == 1, list(out)
+    _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=7 * m + n, sigma_ab=0.05)
+
+
+@pytest.mark.parametrize("m,k,n", [
     (192, 2560, 8192), (256, 4096, 2560), (257, 4096, 2560), (300, 2560, 2560), (320, 4096, 2560), (320, 2560, 1024),
     (321, 2560, 1024),
 ])
