@@ -430,6 +430,7 @@ struct MidPlan {
     bool ok = false;
     int KS = 1, GS = 0, waves = 0, pairs = 1;
     float cost = 0.f;
+    bool fold = true;  // with adapters: the projection in the launch's first blocks (where the launch can)
 };
 struct GemmPlan {
     bool prefill = false;
@@ -501,7 +502,22 @@ void plan_as_prefill(int m, int n, int k, int cus, int thread_k, int thread_n, G
 // on large ones it falls behind from 160 rows on (14336 -> 4096: 55 against 47 us; gate+up 42.5 against 35.2).
 constexpr int kMidMinM = 17, kMidMinMWideShortK = 21, kMidMaxM = 128, kMidMaxMSmallest = 320, kMidMaxMTiny = 512, kMidMaxMVerySmallest = 1024;
 int mid_min_rows(int n, int k, bool lora) { return !lora && k <= 3072 && n >= 10240 ? kMidMinMWideShortK : kMidMinM; }
+static int mid_max_rows_by_weights(int n, int k, bool lora);
 int mid_max_rows(int n, int k, bool lora) {
+    int rows = mid_max_rows_by_weights(n, k, lora);
+    // Wide outputs of a short K: the kernel's time there is its blocks' starts, meetings and stores, one set per
+    // 64 rows and pair of tiles, and the matrix-core kernel's wider blocks overtake it at about 2.1 M (K < 1536) or
+    // 3.2 M output elements whatever the weights' size (896 -> 9728, 8.7 M weights: 13.3 us at 192 rows against 16.3,
+    // but 19.5 / 28.0 / 36.4 at 256 / 384 / 512 against 16.2 / 17.2 / 22.1; 1536 -> 17920 at 192 rows 31.7 against
+    // 23.1; 3584 -> 37888 at 96 / 128 rows 58 / 70 against 56 / 57, with adapters 81 / 97 against 58; while
+    // 2560 -> 12288 and 2048 -> 11264 at 256 rows lead by 9 %: 31.8 against 35.0, 26.9 against 29.6)
+    if (k < 4096) {
+        const int cap = (int)((k < 1536 ? 2100000ll : 3200000ll) / n / 64 * 64);
+        rows = std::min(rows, std::max(cap, mid_max_rows_per_run()));
+    }
+    return rows;
+}
+static int mid_max_rows_by_weights(int n, int k, bool lora) {
     const long long kn = (long long)k * n;
     // the very smallest: to 1024 rows (1024 -> 1024 at 640...1024 rows 6.4...6.6 us against 13.4...14.6 on the
     // matrix-core kernel, 1536 -> 1536 8.7...11.3 against 17...18.5, 2560 -> 1024 11.8...14.6 against 18.5...20; at 4 M
@@ -630,7 +646,18 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
          (!prefill_pinned && g_tune.prefill_min_m == 0 && m >= mid_min_rows(n, k, lora != 0) && m <= mid_max_rows(n, k, lora != 0)))) {
         // with adapters the projection runs in the launch's first blocks: plan for the chip less those
         const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
-        const MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus, lora != 0);
+        MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus, lora != 0);
+        // ... unless the plan for the whole chip is ahead by more than the projection's own launch costs (3 us: what
+        // calls of one plan either way differ by) -- where the product's blocks just fill the chip, the producers push
+        // the plan into another round or another shape: 2560 -> 12288 with two adapters at 128 rows, 128 blocks
+        // of three pairs per run, 26.6 us folded against 22.7 in front; 3584 -> 37888 at 96 rows 81 against 68
+        if (producers > 0 && cus > 2 * producers && g_tune.lora_fold != 2) {
+            MidPlan whole = plan_mid(m, n, k, cus, true);
+            if (whole.ok && (!mp.ok || whole.cost + 3.0f < mp.cost)) {
+                whole.fold = false;
+                mp = whole;
+            }
+        }
         if (mp.ok) {
             gp->mid = true;
             gp->mp = mp;
@@ -895,7 +922,7 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
             folded.lora_adapters = lora->n_adapters;
             // (what the launch itself checks: beyond four runs of rows, or more (slice, tile) words than a copy
             // holds, the projection runs in front -- a call of 320 rows with adapters was refused here once)
-            if (g_tune.lora_fold != 0 && lora->n_adapters <= 8 && mid_lora_fold_ok(folded)) {
+            if (g_tune.lora_fold != 0 && gp.mp.fold && lora->n_adapters <= 8 && mid_lora_fold_ok(folded)) {
                 int end = 0;
                 for (int i = 0; i < 8; ++i) {
                     if (i < lora->n_adapters) end += lora->ranks[i];

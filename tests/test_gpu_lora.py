@@ -60,6 +60,13 @@ def test_lora_on_few_rows_of_other_models_weights(oracle, m, k, n):
     _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=5 * m + n, sigma_ab=0.05)
 
 
+@pytest.mark.parametrize("m,k,n", [(128, 2560, 12288), (100, 2048, 11264), (64, 2560, 12288)])
+def test_lora_where_the_mid_m_blocks_just_fill_the_chip(oracle, m, k, n):
+    """Two runs of 128 three-pair blocks are one round of the chip: the projection's blocks would push the plan
+    into a second round, so it runs in front there (and inside the launch at 64 rows, where there is room)."""
+    _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=11 * m + n, sigma_ab=0.05)
+
+
 @pytest.mark.parametrize("m", [17, 32, 48, 64, 100, 128])
 @pytest.mark.parametrize("k,n", [(11008, 512), (8960, 256)])
 def test_lora_with_a_shorter_last_k_slice(oracle, m, k, n):
