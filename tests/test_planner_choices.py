@@ -73,6 +73,10 @@ def test_sixteen_wavefronts_only_where_twelve_cannot_form_the_plan():
     (320, 4096, 2560, "mid"), (321, 4096, 2560, "matrix-core"), (320, 2560, 1024, "mid"),
     (1024, 2560, 1024, "mid"), (1025, 2560, 1024, "matrix-core"), (512, 3072, 3072, "mid"), (448, 2048, 2048, "mid"),
     (513, 2048, 2048, "matrix-core"), (1024, 1536, 1536, "mid"),
+    # wide outputs of a short K: by output size
+    (192, 896, 9728, "mid"), (193, 896, 9728, "matrix-core"), (384, 896, 4864, "mid"), (448, 896, 4864, "matrix-core"),
+    (128, 1536, 17920, "mid"), (129, 1536, 17920, "matrix-core"), (64, 3584, 37888, "mid"), (65, 3584, 37888, "matrix-core"),
+    (256, 2048, 11264, "mid"), (256, 1024, 8192, "mid"), (257, 1024, 8192, "matrix-core"),
 ])
 def test_which_kernel_takes_a_row_count(m, k, n, want):
     assert _route(m, k, n)[0] == want
