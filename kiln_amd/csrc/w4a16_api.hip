@@ -276,7 +276,11 @@ bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) 
     const int G = k / kGroupK, NT = n / kTileN;
     if (lora && g_tune.lora_fold != 0) cus -= lora_project_slices(m, k);
     const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
-    static const int kWaves[] = {12, 16, 8};
+    // (with adapters a block has one wavefront more, so 14 stand in for the 16 -- 15 main wavefronts and the low-rank
+    // term's operands do not fit LDS at 16 rows: 5120 -> 13824 with two adapters in one round of four-tile blocks
+    // 10.6 / 12.7 us at 1 / 16 rows against 14.3 / 18.0 in two rounds of two-tile blocks, 5120 -> 27648 20.4 / 23.3 against 26.8 / 29.2)
+    const int most = lora ? 14 : 16;
+    const int kWaves[] = {12, most, 8};
     float best_cost = -1.f;
     for (int ks = 1; ks <= kMaxKSlices && ks <= G; ++ks) {
         if (G % ks != 0) continue;
@@ -289,7 +293,7 @@ bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) 
                 // 8.4 us at one row against 10.4 in two rounds of two-tile blocks); elsewhere they
                 // measured 5 to 15 % slower than 12 on the same tiles and slices
                 DecodePlan p;
-                if (waves == 16 && (T != 1 || GS % 16 != 0) && gmp_plan(m, n, k, T, 12, ks, lora, &p)) continue;
+                if (waves == most && (lora || T != 1 || GS % 16 != 0) && gmp_plan(m, n, k, T, 12, ks, lora, &p)) continue;
                 if (!gmp_plan(m, n, k, T, waves, ks, lora, &p)) continue;
                 const int rounds = ceil_div(ceil_div(NT, T) * ks, cus);
                 // The exchange: through counters 0.4 us per slice + 1.2; with the parts as their own
