@@ -317,7 +317,7 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     if constexpr (FOLD) id -= pf.producers;
     [[maybe_unused]] const int consumer = id;
     const int n_blocks = N / BN;
-    const int die_cols = 8 / die_rows, rows_per_die = m_blocks / die_rows;
+    const int die_cols = 8 / die_rows, rows_per_die = (m_blocks + die_rows - 1) / die_rows;
     const int per_die_full = rows_per_die * ((nb_full + die_cols - 1) / die_cols);
     const bool sliced = id >= 8 * per_die_full;
     if (sliced) id -= 8 * per_die_full;
@@ -325,13 +325,13 @@ __global__ __launch_bounds__(64 * WM * NWN, (WM == 2 && NWN == 4) ? 1 : 2) void 
     const int units_per_die = (units + die_cols - 1) / die_cols;
     const int die = id & 7, seq = id >> 3;
     const int unit = (die / die_rows) * units_per_die + seq / rows_per_die;
-    if (seq >= rows_per_die * units_per_die || unit >= units) {  // grid padding (whole block, before any barrier)
+    const int mb = (die % die_rows) * rows_per_die + seq % rows_per_die;
+    if (seq >= rows_per_die * units_per_die || unit >= units || mb >= m_blocks) {  // grid padding (whole block, before any barrier)
         if constexpr (FOLD) {
             if (wave == 0) prefill_fold_done(pf, consumer, lane);  // counted like the others: it will never look
         }
         return;
     }
-    const int mb = (die % die_rows) * rows_per_die + seq % rows_per_die;
     int nb = unit, ks = 0;
     if (sliced) {
         nb = nb_full + unit / KS;
@@ -849,18 +849,35 @@ size_t prefill_lora_t_bytes(int m, bool few_rows) {
     return many;
 }
 
-// Rows of the die grid: the largest power of two up to 8 that divides the row blocks, so that
-// every die owns the same number of them.
-static int prefill_die_rows(int m_blocks) {
-    int dr = 8;
-    while (m_blocks % dr) dr >>= 1;
-    return dr;
+// Rows of the die grid (a power of two up to 8; the dies form rows x 8 / rows over row blocks x units): the one
+// under which the busiest die has the least to do -- ceil(row blocks / rows) row blocks of ceil(units / columns)
+// units each, a whole tile counting as `ks` slices -- and of equals the one with the most rows, so that a die
+// keeps few row blocks of A in its L2.  Neither count need divide: the grid is padded with blocks that leave at once.
+// (Until the row blocks could be padded it was the largest power of two that divides them, i.e. one row of
+// eight columns for any odd count, which leaves dies idle wherever the units are fewer than eight or do not
+// divide by eight: 1024 -> 1024 at 20000 rows, 313 row blocks of three whole column blocks and one more, ran
+// 165 us on three dies and then one, against 58 us at 19968 rows.)
+static int prefill_die_rows(int m_blocks, int units_full, int units_sliced, int ks) {
+    int best = 1;
+    long best_work = -1;
+    for (int dr = 8; dr >= 1; dr >>= 1) {
+        const int dc = 8 / dr, rows = (m_blocks + dr - 1) / dr;
+        const long work = (long)rows * ((long)((units_full + dc - 1) / dc) * ks + (units_sliced + dc - 1) / dc);
+        if (best_work < 0 || work < best_work) {
+            best = dr;
+            best_work = work;
+        }
+    }
+    return best;
+}
+static int prefill_die_rows(int m_blocks, int n, const PrefillPlan &p) {
+    return prefill_die_rows(m_blocks, p.nb_full, (n / p.bn - p.nb_full) * p.ks, p.ks);
 }
 
 // blocks launched: whole tiles, then (tile, K slice) units, each part padded to the die grid
 int prefill_grid(int m, int n, const PrefillPlan &p) {
     const int m_blocks = (m + p.bm - 1) / p.bm;
-    const int dr = prefill_die_rows(m_blocks), dc = 8 / dr, rows = m_blocks / dr;
+    const int dr = prefill_die_rows(m_blocks, n, p), dc = 8 / dr, rows = (m_blocks + dr - 1) / dr;
     const int units_full = p.nb_full, units_sliced = (n / p.bn - p.nb_full) * p.ks;
     return 8 * rows * ((units_full + dc - 1) / dc) + 8 * rows * ((units_sliced + dc - 1) / dc);
 }
@@ -883,8 +900,8 @@ static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm, 
     for (int ks = 2; ks <= 8 && G / ks >= 3; ++ks) {
         const int gsb = (G + ks - 1) / ks;
         if ((ks - 1) * gsb >= G) continue;  // would leave an empty slice
-        const int dr = prefill_die_rows(m_blocks), dc = 8 / dr;
-        if (8 * (m_blocks / dr) * ((rest * ks + dc - 1) / dc) <= sliced_units) p.ks = ks;
+        const int dr = prefill_die_rows(m_blocks, p.nb_full, rest * ks, ks), dc = 8 / dr;
+        if (8 * ((m_blocks + dr - 1) / dr) * ((rest * ks + dc - 1) / dc) <= sliced_units) p.ks = ks;
     }
     return p;
 }
@@ -1015,7 +1032,8 @@ hipError_t launch_shape_as(const PrefillArgs &a, int grid, int m_blocks, int RP,
     w4a16_prefill_kernel<NWN, WM, MI, SWIGLU, RS, FOLD><<<grid + (FOLD ? pf.producers : 0), 64 * NW, lds_bytes, stream>>>(
         (const uint16_t *)a.A, (const u32x4 *)a.B, (const uint16_t *)a.S, (uint16_t *)a.C, (const u32x4 *)a.aext,
         a.M, a.N, a.K, a.Gs, m_blocks, (const uint16_t *)a.lora_t, (const uint16_t *)a.lora_b, a.r_total, RP,
-        a.nb_full, KS, GSb, a.partial, a.counters, prefill_die_rows(m_blocks), pf);
+        a.nb_full, KS, GSb, a.partial, a.counters,
+        prefill_die_rows(m_blocks, a.nb_full, (a.N / (NWN * 64) - a.nb_full) * KS, KS), pf);
     return hipGetLastError();
 }
 

@@ -351,6 +351,10 @@ def test_wrapper_argument_checks_on_device():
     (200, 4096, 2560, 128, 1.0), (512, 2560, 8192, 128, 0.5), (129, 9216, 2560, 128, 0.5),
     (1000, 2560, 2560, 128, 0.5),
     (700, 2560, 8192, 128, 0.5),    # 64-row blocks with the row-sum pre-pass (large launch)
+    # row blocks that no power of two divides, on outputs of few column blocks: the grid over the eight dies is
+    # padded in both directions (5, 9, 11, 21 and 79 row blocks; 2, 3, 4 and 10 column blocks)
+    (300, 512, 768, 128, 0.5), (577, 1024, 1024, 128, 0.5), (700, 256, 512, 128, 0.5), (1300, 1024, 768, 128, 0.5),
+    (1100, 2560, 2560, 128, 0.5), (5000, 256, 1024, 128, 0.5),
 ])
 def test_prefill_cases(oracle, matrix_core_kernel_from_33_rows, m, k, n, g, sigma):
     x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=m * 7 + k + n, sigma=sigma)
