@@ -894,14 +894,25 @@ static PrefillPlan plan_for_shape(int m, int n, int k, int cus, int bn, int bm, 
     p.bm = bm;
     const int G = k / kGroupK, m_blocks = (m + bm - 1) / bm;
     const int n_blocks = n / bn, tiles = m_blocks * n_blocks;
-    p.nb_full = ((tiles / cus) * cus) / m_blocks;  // whole column blocks that fit the whole rounds
+    const int rounds = tiles / cus;
+    p.nb_full = (rounds * cus) / m_blocks;  // whole column blocks that fit the whole rounds
     if (p.nb_full > n_blocks) p.nb_full = n_blocks;
-    const int rest = n_blocks - p.nb_full;
-    for (int ks = 2; ks <= 8 && G / ks >= 3; ++ks) {
-        const int gsb = (G + ks - 1) / ks;
-        if ((ks - 1) * gsb >= G) continue;  // would leave an empty slice
-        const int dr = prefill_die_rows(m_blocks, p.nb_full, rest * ks, ks), dc = 8 / dr;
-        if (8 * ((m_blocks + dr - 1) / dr) * ((rest * ks + dc - 1) / dc) <= sliced_units) p.ks = ks;
+    // ... on every die: the dies deal the tiles as a grid (prefill_die_rows), and a die whose rectangle holds more
+    // whole tiles than its share of the rounds runs a round of its own behind them (4096 -> 4096 at 1100 rows: 18
+    // row blocks x 14 column blocks are 252 tiles, but 36 on each of six dies of 32 units -- 80 us, against 62 us at
+    // 1217 rows, whose 20 x 12 are 30 per die)
+    for (;; --p.nb_full) {
+        const int rest = n_blocks - p.nb_full;
+        p.ks = 1;
+        for (int ks = 2; ks <= 8 && G / ks >= 3; ++ks) {
+            const int gsb = (G + ks - 1) / ks;
+            if ((ks - 1) * gsb >= G) continue;  // would leave an empty slice
+            const int dr = prefill_die_rows(m_blocks, p.nb_full, rest * ks, ks), dc = 8 / dr;
+            if (8 * ((m_blocks + dr - 1) / dr) * ((rest * ks + dc - 1) / dc) <= sliced_units) p.ks = ks;
+        }
+        if (p.nb_full == 0 || p.nb_full == n_blocks) break;
+        const int dr = prefill_die_rows(m_blocks, p.nb_full, rest * p.ks, p.ks), dc = 8 / dr;
+        if (((m_blocks + dr - 1) / dr) * ((p.nb_full + dc - 1) / dc) <= rounds * (cus / 8)) break;
     }
     return p;
 }
