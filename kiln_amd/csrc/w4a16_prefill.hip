@@ -1206,7 +1206,27 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         int rb = 0, row_tiles = 0, kz = 0, per_slice = 0;
         project_slicing(a.M, a.K, a.counters != nullptr, &rb, &row_tiles, &kz, &per_slice);
         const int sliced_tiles = (a.N / a.bn - a.nb_full) * ((a.M + a.bm - 1) / a.bm);
-        fold = a.lora_words && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
+        // A product that fits the chip's block slots in one go must still fit them with the projection's blocks
+        // in front: the blocks that find no slot start when the producers leave, on whichever units the
+        // dispatcher picks, and two of them on one unit beside idle units take 1.6 times as long as one (4096 ->
+        // 4096 at 1700 rows, 224 blocks of 128 x 256 and 328 producers for 512 slots: 121 us against 86 at 1600
+        // rows, 300 + 208 blocks; 97 with the projection in front).  So the projection is cut into fewer K slices
+        // there -- its blocks stay far shorter than the product's -- and runs in front if its row tiles alone do
+        // not fit.  Launches of several rounds keep all slices (gate+up at 2048 rows 189 us inside, 194 in front).
+        bool room = true;
+        if (rb == 16 && (a.bm == 64 || a.bm == 128)) {
+            const int slots = a.cus * (a.bm == 128 ? 2 : 3), product = prefill_grid(a.M, a.N, shape);
+            if (product <= slots && product + (row_tiles * kz + 7) / 8 * 8 > slots) {
+                const int cap = (slots - product) / 8 * 8 / row_tiles;
+                room = cap >= 1;
+                if (room) {
+                    const int steps = a.K / 32;
+                    per_slice = ((steps + cap - 1) / cap + 3) / 4 * 4;
+                    kz = (steps + per_slice - 1) / per_slice;
+                }
+            }
+        }
+        fold = room && a.lora_words && a.bn == 256 && (a.bm == 64 || a.bm == 128) && rb == 16 &&
                a.counters && row_tiles <= kPrefillFoldMaxTiles && row_tiles <= kProjectMaxCounters - kProjectFoldCounters &&
                sliced_tiles <= kProjectFoldCounters && a.n_adapters >= 1 && a.n_adapters <= 8 && a.lora_a && a.lora_t &&
                a.ranks && a.scales && a.r_total <= kProjectMaxRank;

@@ -38,6 +38,9 @@ def _lora_case(oracle, m, k, n, ranks, scales, seed, sigma_x=1.0, sigma_ab=0.02)
     (300, 256, 256, (4, 5), (1.0, 3.0)),            # ranks that are not multiples of 8
     (1100, 4224, 256, (16, 32), (0.5, 1.0)),        # long K and many rows: the projection's 64-row blocks
     (200, 9216, 256, (7,), (1.5,)),                 # long K, few row tiles: 16 K slices meet per tile
+    # the product's blocks fit the chip's block slots, but not together with all K slices of the projection in
+    # front of them: the projection is cut into fewer slices
+    (900, 2560, 8192, (16, 32), (0.5, 1.0)), (576, 4096, 4096, (16, 32), (0.5, 1.0)),
 ])
 def test_fused_lora_matches_oracle(oracle, m, k, n, ranks, scales):
     _lora_case(oracle, m, k, n, ranks, scales, seed=m + n)
