@@ -36,11 +36,11 @@ LAYERS = 16
 TIMED_REPLAYS = 5      # of the graph that holds the timed steps; the median replay is reported
 # HBM bytes per launch of the gate+up decode kernel at M=16, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by what the same counter reads for a 64 MiB device
-# copy (x1.9989 and x1.0): 12307.4 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
+# copy (x1.9989 and x1.0): 12307.1 KiB * 1.9989 + 576.0 KiB.  Source: profiles/decode_gmp_kernel_m16_hbm_traffic.txt
 # The counters cannot be read inside an untraced run, so the figure is carried as a constant -- of one
 # kernel instance on one plan: where the planner picks another for the headline shape the line reports no
 # traffic instead of this one.
-GATE_UP_M16_TRAFFIC = {"bytes": 25781555, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
+GATE_UP_M16_TRAFFIC = {"bytes": 25780980, "kernel": "w4a16_decode_gmp_kernel<5, 3, 4, false>", "blocks": 231}
 MIN_TIMED_REGION_S = 0.02   # a timed region shorter than this replays its graph several times between the events
 
 

@@ -1212,10 +1212,12 @@ hipError_t launch_prefill(const PrefillArgs &a, hipStream_t stream) {
         // 4096 at 1700 rows, 224 blocks of 128 x 256 and 328 producers for 512 slots: 121 us against 86 at 1600
         // rows, 300 + 208 blocks; 97 with the projection in front).  So the projection is cut into fewer K slices
         // there -- its blocks stay far shorter than the product's -- and runs in front if its row tiles alone do
-        // not fit.  Launches of several rounds keep all slices (gate+up at 2048 rows 189 us inside, 194 in front).
+        // not fit.  Launches of several rounds keep all slices (gate+up at 2048 rows 189 us inside, 194 in front), and
+        // so do 64-row blocks, three to a unit, which were never seen to suffer (gate+up at 512 rows, 768 blocks and
+        // 256 producers for 768 slots: 62 us inside, 68 in front).
         bool room = true;
-        if (rb == 16 && (a.bm == 64 || a.bm == 128)) {
-            const int slots = a.cus * (a.bm == 128 ? 2 : 3), product = prefill_grid(a.M, a.N, shape);
+        if (rb == 16 && a.bm == 128) {
+            const int slots = a.cus * 2, product = prefill_grid(a.M, a.N, shape);
             if (product <= slots && product + (row_tiles * kz + 7) / 8 * 8 > slots) {
                 const int cap = (slots - product) / 8 * 8 / row_tiles;
                 room = cap >= 1;
