@@ -515,7 +515,9 @@ int mid_max_rows(int n, int k, bool lora) {
     // but 19.5 / 28.0 / 36.4 at 256 / 384 / 512 against 16.2 / 17.2 / 22.1; 1536 -> 17920 at 192 rows 31.7 against
     // 23.1; 3584 -> 37888 at 96 / 128 rows 58 / 70 against 56 / 57, with adapters 81 / 97 against 58; while
     // 2560 -> 12288 and 2048 -> 11264 at 256 rows lead by 9 %: 31.8 against 35.0, 26.9 against 29.6)
-    if (k < 4096) {
+    // (K = 4096 included: 4096 -> 28672 at 128 rows 68 us against 58 on the matrix-core kernel, with two adapters 78
+    // against 56, while 4096 -> 22016, 2.8 M output elements there, leads with 49 against 67)
+    if (k <= 4096) {
         const int cap = (int)((k < 1536 ? 2100000ll : 3200000ll) / n / 64 * 64);
         rows = std::min(rows, std::max(cap, mid_max_rows_per_run()));
     }

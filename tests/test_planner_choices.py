@@ -77,6 +77,7 @@ def test_sixteen_wavefronts_only_where_twelve_cannot_form_the_plan():
     (192, 896, 9728, "mid"), (193, 896, 9728, "matrix-core"), (384, 896, 4864, "mid"), (448, 896, 4864, "matrix-core"),
     (128, 1536, 17920, "mid"), (129, 1536, 17920, "matrix-core"), (64, 3584, 37888, "mid"), (65, 3584, 37888, "matrix-core"),
     (256, 2048, 11264, "mid"), (256, 1024, 8192, "mid"), (257, 1024, 8192, "matrix-core"),
+    (64, 4096, 28672, "mid"), (65, 4096, 28672, "matrix-core"), (128, 4096, 22016, "mid"),
 ])
 def test_which_kernel_takes_a_row_count(m, k, n, want):
     assert _route(m, k, n)[0] == want
