@@ -56,9 +56,9 @@ typedef int kiln_marlin_status_t;
  * waiting block only waits for lower indices, so a launch that has the GPU to itself always gets there.
  */
 #define KILN_W4A16_WAIT_DECODE_EXCHANGE 1u   /* K slices of a call of up to 16 rows */
-#define KILN_W4A16_WAIT_MID_EXCHANGE    2u   /* K slices of a call of 17...320 rows */
+#define KILN_W4A16_WAIT_MID_EXCHANGE    2u   /* K slices of a call the mid-M kernel takes (17 rows up to 1024) */
 #define KILN_W4A16_WAIT_DECODE_FOLD     4u   /* LoRA projection inside a launch of up to 16 rows */
-#define KILN_W4A16_WAIT_MID_FOLD        8u   /* ... of 17...320 rows */
+#define KILN_W4A16_WAIT_MID_FOLD        8u   /* ... of 17...320 rows on the mid-M kernel */
 #define KILN_W4A16_WAIT_PREFILL_FOLD    16u  /* ... on the matrix-core path */
 
 /* Size of the static device array behind kiln_marlin_w4a16_gemm_static_scratch (per GPU). */

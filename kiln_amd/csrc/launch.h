@@ -24,9 +24,9 @@ constexpr size_t kWsFoldFlagOffset = kWsCounterBytes + kWsFlaggedBytes - kWsFold
 constexpr size_t kWsZeroedBytes = kWsCounterBytes + kWsFlaggedBytes;
 enum WaitGaveUp : unsigned {
     kGaveUpDecodeExchange = 1u,  // K slices of a launch of up to 16 rows
-    kGaveUpMidExchange = 2u,     // K slices of a launch of 17...320 rows
+    kGaveUpMidExchange = 2u,     // K slices of a launch of the mid-M kernel (17 rows up to 1024)
     kGaveUpDecodeFold = 4u,      // a block of up to 16 rows waiting for the folded LoRA projection
-    kGaveUpMidFold = 8u,         // the same at 17...320 rows
+    kGaveUpMidFold = 8u,         // the same in a launch of the mid-M kernel with adapters (17...320 rows)
     kGaveUpPrefillFold = 16u,    // the same on the matrix-core path
 };
 
