@@ -220,6 +220,40 @@ def test_proj_forward_and_merge_concat(oracle):
     assert torch.allclose(ba, want, atol=1e-5)
 
 
+def test_host_mirror_pads_odd_stacked_ranks():
+    """Ranks 4 and 5 through `proj_forward` and `swiglu_forward`: the mirror pads the stacked rank to a multiple of 8
+    (zero rows of A, zero columns of B), and the result equals the unpadded call through the library's general route."""
+    k, n = 2560, 512
+    b = torch.randint(-2**31, 2**31 - 1, (k // 16, 2 * n), dtype=torch.int32, device="cuda")
+    s = (torch.rand(k // 128, n, device="cuda") * 0.018 + 0.002).half()
+    proj = marlin_proj.MarlinPackedProj(b, s, 128, k, n)
+    p1 = klora.LoraProjectionWeights((torch.randn(4, k, device="cuda") * 0.05).bfloat16(), (torch.randn(n, 4, device="cuda") * 0.05).bfloat16())
+    p2 = klora.LoraProjectionWeights((torch.randn(5, k, device="cuda") * 0.05).bfloat16(), (torch.randn(n, 5, device="cuda") * 0.05).bfloat16())
+    stacked = klora.stack_adapters([p1, p2], [0.5, 2.0])
+    assert klora.pad_rank(stacked).ranks == (4, 12)
+    for m in (3, 16, 40, 200):
+        x = torch.randn(m, k, device="cuda").bfloat16()
+        unpadded = marlin_gemm.marlin_w4a16_gemm_lora(x, b, s, 128, stacked.a_cat, stacked.b_cat, stacked.ranks, stacked.scales)
+        y = klora.proj_forward(x, proj, stacked)
+        ref = x.float() @ marlin_gemm.dequant_f32(b, s, 128)
+        for p, sc in ((p1, 0.5), (p2, 2.0)):
+            ref = ref + (sc * (x.float() @ p.a.float().T)).bfloat16().float() @ p.b.float().T
+        tol = 2e-2 * ref.abs().max()
+        assert (y.float() - ref).abs().max() <= tol and (unpadded.float() - ref).abs().max() <= tol
+    # the fused gate/up call: 256 gate + 256 up columns, rank 4 on the gate side and 5 on the up side
+    half = n // 2
+    g = klora.LoraProjectionWeights(p1.a, p1.b[:half].contiguous())
+    u = klora.LoraProjectionWeights(p2.a, p2.b[:half].contiguous())
+    x = torch.randn(16, k, device="cuda").bfloat16()
+    h = klora.swiglu_forward(x, proj, g, u, 1.0)
+    z = x.float() @ marlin_gemm.dequant_f32(b, s, 128)
+    v = z.view(16, n // 16, 2, 8)
+    gate = v[:, :, 0].reshape(16, half) + (x.float() @ g.a.float().T).bfloat16().float() @ g.b.float().T
+    up = v[:, :, 1].reshape(16, half) + (x.float() @ u.a.float().T).bfloat16().float() @ u.b.float().T
+    want = torch.nn.functional.silu(gate) * up
+    assert (h.float() - want).abs().max() <= 2e-2 * want.abs().max()
+
+
 def test_lora_argument_errors():
     dev = "cuda"
     a = torch.zeros(2, 128, dtype=torch.bfloat16, device=dev)

@@ -554,5 +554,15 @@ def test_adapters_of_side_by_side_projections_become_one_block_structured_set():
     assert torch.allclose(delta[:48], want_q, rtol=1e-5, atol=1e-5) and torch.count_nonzero(delta[48:64]) == 0
     assert torch.allclose(delta[64:], 3.0 * (v.b.float() @ v.a.float()), rtol=1e-5, atol=1e-5)
     assert fuse_column_blocks([None, None], (8, 8)) is None
+    # pad_rank: zero rows of A and zero columns of B up to a multiple of 8, the delta unchanged
+    from kiln_amd.lora import pad_rank
+    odd = stack_adapters([mk(48, 4), mk(48, 5)], [0.5, 2.0])
+    padded = pad_rank(odd)
+    assert padded.ranks == (4, 12) and tuple(padded.a_cat.shape) == (16, k) and tuple(padded.b_cat.shape) == (48, 16)
+    assert torch.equal(padded.a_cat[:9], odd.a_cat) and torch.count_nonzero(padded.a_cat[9:]) == 0
+    assert torch.equal(padded.b_cat[:, :9], odd.b_cat) and torch.count_nonzero(padded.b_cat[:, 9:]) == 0
+    assert pad_rank(padded) is padded and pad_rank(q) is not q and pad_rank(fused) is fused
+    big = stack_adapters([mk(48, 61)], [1.0])
+    assert pad_rank(big).ranks == (64,) and pad_rank(stack_adapters([mk(48, 30), mk(48, 35)], [1.0, 1.0])).ranks == (30, 35)
     with pytest.raises(marlin_proj.MarlinProjError):
         fuse_column_blocks([v, None], (48, 16))
