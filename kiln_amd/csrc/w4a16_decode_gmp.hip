@@ -529,6 +529,16 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             // adds all parts in ascending K order (so the result does not depend on arrival order)
             // and leaves the counter zero
             KILN_GMP_TL(3, KILN_GMP_NOW());
+            // With adapters the last slice's part carries the low-rank term: whichever slice arrives last finishes the
+            // tile here, and only the last slice's blocks hold the term's operands (adds_term).  (Added behind the
+            // exchange instead, the term came from LDS that nobody had filled whenever another slice arrived last:
+            // always, with the slices of a tile on compute units of one round.)
+            if constexpr (LORA) {
+                if (adds_term) {
+                    lds_signal_wait(lora_ready_addr(), kGmpOperandsReady);  // the term's operands are in LDS
+                    lora_add_from_lds(sum, lo, lora_t_lds, lora_b_lds, ti, M, lane);
+                }
+            }
             float *dst = partial + ((size_t)ks * NT + tt) * 256 + lane * 4;
 #pragma unroll
             for (int i = 0; i < 4; ++i) __hip_atomic_store(dst + i, sum[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -549,7 +559,7 @@ __global__ __launch_bounds__(kGmpMaxWaves * 64) void w4a16_decode_gmp_kernel(
             }
             KILN_GMP_TL(4, KILN_GMP_NOW());
         }
-        if (adapter) {
+        if (adapter && (KS == 1 || flagged)) {  // (through counters it is in the last slice's part already)
             lds_signal_wait(lora_ready_addr(), kGmpOperandsReady);  // the term's operands are in LDS
             lora_add_from_lds(sum, lo, lora_t_lds, lora_b_lds, ti, M, lane);
         }

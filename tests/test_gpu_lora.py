@@ -220,6 +220,44 @@ def test_proj_forward_and_merge_concat(oracle):
     assert torch.allclose(ba, want, atol=1e-5)
 
 
+@pytest.mark.parametrize("tiles,waves,ks", [(2, 12, 3), (1, 12, 6), (1, 12, 2), (3, 12, 4)])
+@pytest.mark.parametrize("m", [16, 5])
+def test_lora_with_the_k_slices_meeting_through_counters(oracle, tiles, waves, ks, m):
+    """Forced plans of the small-M kernel on the down projection with the counter-free exchange switched off (and six
+    slices, which are beyond it anyway): whichever slice arrives last finishes a tile, so the low-rank term travels in
+    the last slice's part.  20 calls each: the slices of a tile run side by side and arrive in any order."""
+    from kiln_amd import _lib
+    L = _lib.load_tuning()
+    L.kiln_w4a16_debug_gmp(tiles, waves, ks)
+    L.kiln_w4a16_debug_flagged(0)
+    k, n, g = 9216, 2560, 128
+    x, q, s_bits = oracle.gen_problem(m, k, n, g, seed=31 * m + ks)
+    b, s = pack.repack_gptq(q, s_bits, None, g)
+    ranks, scales = (16, 32), (0.5, 1.0)
+    a_list = [oracle.gen_normal_bf16(r, k, 0.05, seed=40 + i) for i, r in enumerate(ranks)]
+    b_list = [oracle.gen_normal_bf16(n, r, 0.05, seed=50 + i) for i, r in enumerate(ranks)]
+    y_ref = oracle.c_w4a16_cpu_path(x, q, s_bits, g)
+    for a_i, b_i, sc in zip(a_list, b_list, scales):
+        oracle.c_lora_delta_add(y_ref, x, a_i, b_i, sc)
+    bt, st = upload_packed(b, s)
+    a_cat, b_cat = bf16_tensor(np.concatenate(a_list, axis=0)), bf16_tensor(np.concatenate(b_list, axis=1))
+    first = None
+    for _ in range(20):
+        y = marlin_gemm.marlin_w4a16_gemm_lora(bf16_tensor(x), bt, st, g, a_cat, b_cat, ranks, scales)
+        torch.cuda.synchronize()
+        first = y if first is None else first
+        assert torch.equal(y, first), "the result depends on the order in which the slices arrive"
+    err, _, _ = row_errors(bf16_bits(first), y_ref, oracle)
+    assert err.max() <= 1e-2, f"worst row error {err.max():.3e}"
+
+
+def test_lora_on_an_output_too_wide_for_the_counter_free_exchange(oracle):
+    """21760 columns in three K slices are more partial tiles than the zeroed region holds: the automatic plan meets
+    through counters, in a launch of several rounds of blocks (a random sweep found NaNs here)."""
+    for _ in range(3):
+        _lora_case(oracle, 14, 9216, 21760, (32, 32), (1.0, 1.0), seed=63, sigma_ab=0.03)
+
+
 def test_host_mirror_pads_odd_stacked_ranks():
     """Ranks 4 and 5 through `proj_forward` and `swiglu_forward`: the mirror pads the stacked rank to a multiple of 8
     (zero rows of A, zero columns of B), and the result equals the unpadded call through the library's general route."""
