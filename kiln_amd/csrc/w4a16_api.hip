@@ -274,7 +274,8 @@ bool flagged_exchange_fits(int ks, int n) {
 // that project x onto the adapters, so that the projection can ride in the same launch.
 bool plan_decode_gmp(int m, int n, int k, int cus, bool lora, DecodePlan *best) {
     const int G = k / kGroupK, NT = n / kTileN;
-    if (lora && g_tune.lora_fold != 0) cus -= lora_project_slices(m, k);
+    // (a caller may name a part of the chip, `sms`: never plan for less than one unit)
+    if (lora && g_tune.lora_fold != 0 && cus > lora_project_slices(m, k)) cus -= lora_project_slices(m, k);
     const int a_kib_per_group = m <= 4 ? 1 : (m <= 8 ? 2 : 4);
     // (with adapters a block has one wavefront more, so 14 stand in for the 16 -- 15 main wavefronts and the low-rank
     // term's operands do not fit LDS at 16 rows: 5120 -> 13824 with two adapters in one round of four-tile blocks

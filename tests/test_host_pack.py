@@ -566,3 +566,19 @@ def test_adapters_of_side_by_side_projections_become_one_block_structured_set():
     assert pad_rank(big).ranks == (64,) and pad_rank(stack_adapters([mk(48, 30), mk(48, 35)], [1.0, 1.0])).ranks == (30, 35)
     with pytest.raises(marlin_proj.MarlinProjError):
         fuse_column_blocks([v, None], (48, 16))
+
+
+def test_workspace_sizing_for_a_part_of_the_chip():
+    """`sms` may name fewer compute units than the projection of a call with adapters would take for itself (eight
+    at K = 4096): the planners never plan for less than one unit.  In a child process: the failure was a division
+    by zero on the host, which ends the process."""
+    import os, subprocess, sys
+    code = ("from kiln_amd import _lib\n"
+            "L = _lib.load()\n"
+            "for m, n, k, sms in [(129, 9216, 4096, 8), (24, 18432, 384, 1), (16, 2560, 9216, 3), (2048, 18432, 2560, 2), (64, 2560, 4096, 5)]:\n"
+            "    v = L.kiln_w4a16_workspace_bytes_tuned(m, n, k, -1, -1, sms)\n"
+            "    assert 0 < v < 1 << 31, (m, n, k, sms, v)\n"
+            "print('sized')\n")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    r = subprocess.run([sys.executable, "-c", code], cwd=root, capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0 and "sized" in r.stdout, (r.returncode, r.stderr[-500:])
