@@ -111,3 +111,78 @@ def test_random_shapes_through_every_entry(seed, boundary):
             worst.append((err, case))
         torch.cuda.empty_cache()
     assert not worst, worst
+
+
+OVERRIDE_K = [128, 256, 512, 1024, 4096]
+OVERRIDE_N = [16, 32, 64, 128, 256]
+UNITS = [1, 8, 40, 64, 104, 128, 200, 256, 304, 512]
+
+
+@pytest.mark.parametrize("seed", [5, 6, 7])
+def test_random_shapes_on_a_workspace_of_exactly_the_size_asked_for(seed):
+    """The same through the C ABI itself, with what the wrappers never pass -- tile overrides and a count of
+    compute units on the plain entry, eight adapters -- on a workspace of exactly `kiln_w4a16_*workspace_bytes`
+    with a canary behind it, called twice without zeroing in between: the result, the canary, and the zeroed prefix
+    that every call must leave as it found it."""
+    import ctypes
+    from kiln_amd import _lib
+    L = _lib.load()
+    rnd = random.Random(seed)
+    torch.manual_seed(seed)
+    stream = torch.cuda.current_stream().cuda_stream
+    zeroed = L.kiln_w4a16_workspace_zeroed_bytes()
+    worst = []
+    for c in range(40):
+        k, n = rnd.choice(MODEL_K + ANY_K), rnd.choice(MODEL_N + ANY_N)
+        m = rnd.choice(BOUNDARY_M + [1, 3, 8, 14, 100, 300, 577, 900, 1100, 1700, 2048])
+        while m * n * k > 1e11:
+            m = max(1, m // 2)
+        g = rnd.choice([128, 128, -1])
+        kind = rnd.choice(["plain", "lora", "swiglu", "swiglu_lora"])
+        if kind.startswith("swiglu") and n % 512 != 0:
+            n += 256
+        ranks = rnd.choice(RANKS + [(8,) * 8])
+        scales = tuple(rnd.choice([0.5, 1.0, 2.0]) for _ in ranks)
+        tk, tn, sms = rnd.choice([-1, -1] + OVERRIDE_K), rnd.choice([-1, -1] + OVERRIDE_N), rnd.choice([-1, -1] + UNITS)
+        case = (kind, m, k, n, g, ranks, scales, tk, tn, sms)
+        print(f"case {c}: {case}", flush=True)
+        b, s = _weights(k, n, g)
+        x = torch.randn(m, k, device="cuda").bfloat16()
+        rt = sum(ranks)
+        la = (torch.randn(rt, k, device="cuda") * 0.03).bfloat16()
+        lb = (torch.randn(n, rt, device="cuda") * 0.03).bfloat16()
+        ref = x.float() @ mg.dequant_f32(b, s, g)
+        if kind in ("lora", "swiglu_lora"):
+            o = 0
+            for r, sc in zip(ranks, scales):
+                ref = ref + (sc * (x.float() @ la[o:o + r].float().T)).bfloat16().float() @ lb[:, o:o + r].float().T
+                o += r
+        n_out = n // 2 if kind.startswith("swiglu") else n
+        if kind.startswith("swiglu"):
+            ref = _swiglu_of(ref)
+        nbytes = (L.kiln_w4a16_workspace_bytes_tuned(m, n, k, tk, tn, sms) if kind == "plain" else
+                  L.kiln_w4a16_workspace_bytes(m, n, k) if kind == "lora" else L.kiln_w4a16_swiglu_workspace_bytes(m, n_out, k))
+        ws = torch.zeros(nbytes + 256, dtype=torch.uint8, device="cuda")
+        ws[nbytes:] = 0x5A
+        y = torch.empty(m, n_out, dtype=torch.bfloat16, device="cuda")
+        cr, cs = (ctypes.c_int * len(ranks))(*ranks), (ctypes.c_float * len(ranks))(*scales)
+        for _ in range(2):
+            ptrs = (x.data_ptr(), b.data_ptr(), y.data_ptr(), s.data_ptr())
+            lora = (la.data_ptr(), lb.data_ptr(), rt, len(ranks), cr, cs)
+            if kind == "plain":
+                st = L.kiln_marlin_w4a16_gemm(*ptrs, m, n, k, ws.data_ptr(), g, 0, stream, tk, tn, sms, 16)
+            elif kind == "lora":
+                st = L.kiln_w4a16_gemm_lora(*ptrs, m, n, k, ws.data_ptr(), g, 0, stream, *lora)
+            elif kind == "swiglu":
+                st = L.kiln_w4a16_gemm_swiglu(*ptrs, m, n_out, k, ws.data_ptr(), g, 0, stream)
+            else:
+                st = L.kiln_w4a16_gemm_swiglu_lora(*ptrs, m, n_out, k, ws.data_ptr(), g, 0, stream, *lora)
+            torch.cuda.synchronize()
+            if st == 2 and kind == "plain" and (tk > 0 or tn > 0):
+                break   # a tile override the shape does not take (ERR_KERN_SHAPE), refused before anything ran
+            err = float("nan") if st else _rel(y, ref)
+            intact = bool((ws[nbytes:] == 0x5A).all()) and int(ws[:zeroed].count_nonzero()) == 0
+            if not (err <= TOL and intact):
+                worst.append((st, err, intact, case))
+        torch.cuda.empty_cache()
+    assert not worst, worst
