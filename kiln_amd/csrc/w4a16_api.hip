@@ -648,9 +648,22 @@ void plan_gemm(int m, int n, int k, int cus, int thread_k, int thread_n, int lor
     // in the launch's first blocks where it fits, else from one launched in front)
     // (a call pinned to a block shape of the matrix-core kernel goes there)
     const bool prefill_pinned = g_tune.prefill_bm != 0 || g_tune.prefill_bn != 0 || g_tune.prefill_ks != 0 || g_tune.prefill_nb_full >= 0;
+    // (with adapters also below 17 rows where the small-M launch would have to take the projection from a launch in
+    // front -- its blocks fill the chip and leave the producers no units of their own -- and this kernel need not:
+    // 11008 -> 4096, 256 blocks of two tiles in two slices, with two adapters 15.3...17.0 us at 1...16 rows, here 13.9...14.4)
+    bool few_rows_here = false;
+    if (lora == 1 && m <= 16 && g_tune.lora_fold != 0 && g_tune.lora_fold != 2 && g_tune.gmp_tiles == 0 && thread_k <= 0 && thread_n <= 0) {
+        DecodePlan dp;
+        if (plan_decode_gmp(m, n, k, cus, true, &dp)) {
+            const int steps = k / 32, kz0 = lora_project_slices(m, k), per = ((steps + kz0 - 1) / kz0 + 3) / 4 * 4;
+            const int kz = (steps + per - 1) / per, blocks = dp.BPS * dp.KS;
+            few_rows_here = blocks <= cus && blocks + kz > cus;
+        }
+    }
     if (lora != 2 && thread_k <= 0 && thread_n <= 0 && g_tune.mid != 0 &&
         (g_tune.mid == 1 ||
-         (!prefill_pinned && g_tune.prefill_min_m == 0 && m >= mid_min_rows(n, k, lora != 0) && m <= mid_max_rows(n, k, lora != 0)))) {
+         (!prefill_pinned && g_tune.prefill_min_m == 0 && (m >= mid_min_rows(n, k, lora != 0) || few_rows_here) &&
+          m <= mid_max_rows(n, k, lora != 0)))) {
         // with adapters the projection runs in the launch's first blocks: plan for the chip less those
         const int producers = lora && g_tune.lora_fold != 0 ? ceil_div(m, 16) * lora_project_slices(m, k) : 0;
         MidPlan mp = plan_mid(m, n, k, cus > 2 * producers ? cus - producers : cus, lora != 0);

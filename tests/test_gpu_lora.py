@@ -58,7 +58,7 @@ def test_lora_on_few_rows(oracle, m, k, n):
     (1, 18944, 3584), (16, 18944, 3584),   # the projection's wavefronts take ten steps of K each
     (5, 5120, 13824), (16, 5120, 13824),   # 40 groups unsliced: 14 main wavefronts of three groups beside the adapter's
     (3, 5120, 27648),                      # ... and a launch of more blocks than compute units, the projection in its first ones
-    (16, 11008, 4096),                     # as many blocks as compute units: the projection runs in front
+    (16, 11008, 4096), (3, 11008, 4096),   # as many small-M blocks as compute units: the mid-M kernel takes the call, from one row
 ])
 def test_lora_on_few_rows_of_other_models_weights(oracle, m, k, n):
     _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=5 * m + n, sigma_ab=0.05)
