@@ -583,7 +583,7 @@ MidPlan plan_mid_waves(int m, int n, int k, int cus, bool lora, bool ten_beyond_
             a.K = k;
             a.KS = ks;
             a.GS = ceil_div(G, ks);  // the last slice may be shorter (mid_plan_ok says when)
-            // Ten wavefronts where a launch may have them (up to 32 rows, or one pair per block; no adapters) and eight
+            // Ten wavefronts where a launch may have them (up to 32 rows, or one pair per block without adapters) and eight
             // would take four groups each or more: 5120 -> 13824 at 17...32 rows 16.7...17.3 us (eight cannot
             // hold 40 groups: two slices) -> 13.0...13.9, 4096 -> 14336 12.0...12.4 -> 11.6...12.0.  Not below:
             // 20 groups as 10 x 2 measured 2...9 % slower than as 4 x 3 + 4 x 2 (in-projection 6.4 -> 6.5 us,
@@ -593,6 +593,10 @@ MidPlan plan_mid_waves(int m, int n, int k, int cus, bool lora, bool ten_beyond_
             // of 10 x 4 against 26.0 in six of 8 x 3; 5120 -> 5120 15.2 against 13.1): there they are the plan of
             // last resort (plan_mid).
             int max_waves = a.GS > 24 && (m <= 32 || ten_beyond_32_rows) ? mid_max_waves(m, pairs, lora) : 8;
+            // (with adapters in plans of one or two slices only: 5120 -> 13824 with two adapters at 17 rows 19.3 -> 15.1 us
+            // unsliced, 9216 -> 2560 13.1 -> 12.0 and 8192 -> 8192 21.0 -> 19.8 in two slices, but 13824 -> 5120 in three
+            // slices of 6 x 4 + 4 x 3 groups 22.2 against 20.0 in four slices of eight wavefronts)
+            if (lora && ks > 2) max_waves = 8;
             if (g_tune.mid_waves > 0) max_waves = std::min(g_tune.mid_waves, mid_max_waves(m, pairs, lora));
             a.waves = a.GS < max_waves ? a.GS : max_waves;
             a.pairs = pairs;

@@ -64,6 +64,13 @@ def test_lora_on_few_rows_of_other_models_weights(oracle, m, k, n):
     _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=5 * m + n, sigma_ab=0.05)
 
 
+@pytest.mark.parametrize("m,k,n", [(17, 5120, 512), (32, 5120, 768), (24, 9216, 512), (32, 8192, 1024), (20, 4096, 512)])
+def test_lora_on_ten_wavefronts(oracle, m, k, n):
+    """Up to 32 rows the blocks of a call with adapters may have ten wavefronts, in plans of one or two K slices:
+    40 and 32 groups unsliced, 72 and 64 in two slices."""
+    _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=13 * m + n, sigma_ab=0.05)
+
+
 @pytest.mark.parametrize("m,k,n", [(128, 2560, 12288), (100, 2048, 11264), (64, 2560, 12288)])
 def test_lora_where_the_mid_m_blocks_just_fill_the_chip(oracle, m, k, n):
     """Two runs of 128 three-pair blocks are one round of the chip: the projection's blocks would push the plan
