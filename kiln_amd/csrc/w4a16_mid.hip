@@ -656,9 +656,9 @@ __device__ __forceinline__ void mid_block(
 constexpr int kMidOneRowBlock = 1, kMidTwoRowBlocks = 2, kMidRowBlocksByRun = 0;
 
 // (one pair per block: 114...153 registers whatever the row blocks, so ten wavefronts there too; with adapters the
-// one-row-block instances of up to two pairs: 162)
+// one-row-block instances: 162...166)
 template <int TP, int ROW_BLOCKS, bool LORA>
-constexpr int kMidWavesOf = (ROW_BLOCKS == kMidOneRowBlock && (!LORA || TP <= 2)) || (!LORA && TP == 1) ? kMidWavesMost : kMidWaves;
+constexpr int kMidWavesOf = ROW_BLOCKS == kMidOneRowBlock || (!LORA && TP == 1) ? kMidWavesMost : kMidWaves;
 
 template <int TP, int GPW, bool LORA, int ROW_BLOCKS>
 __global__ __launch_bounds__((kMidWavesOf<TP, ROW_BLOCKS, LORA> * 64)) void w4a16_mid_kernel(
@@ -781,10 +781,10 @@ bool mid_lora_fold_ok(const MidArgs &a) {
 // makes the tile count even; a last block may hold fewer pairs), equal K slices, at most eight
 // wavefronts of one to four groups each, every wavefront at least one group.
 // Ten wavefronts fit a compute unit's LDS (10 x 16 KiB) and, three to a SIMD, hold at most 170 registers each:
-// the instances of a pass over one row block do (up to 32 rows; with adapters those of up to two pairs per block: 162
+// the instances of a pass over one row block do (up to 32 rows; with adapters 162...166
 // registers), and those of one pair per block without adapters.
 int mid_max_waves(int m, int pairs, bool lora) {
-    if (lora) return m <= 32 && pairs <= 2 ? kMidWavesMost : kMidWaves;
+    if (lora) return m <= 32 ? kMidWavesMost : kMidWaves;
     return m <= 32 || pairs == 1 ? kMidWavesMost : kMidWaves;
 }
 

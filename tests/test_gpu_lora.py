@@ -64,7 +64,8 @@ def test_lora_on_few_rows_of_other_models_weights(oracle, m, k, n):
     _lora_case(oracle, m, k, n, (16, 32), (0.5, 1.0), seed=5 * m + n, sigma_ab=0.05)
 
 
-@pytest.mark.parametrize("m,k,n", [(17, 5120, 512), (32, 5120, 768), (24, 9216, 512), (32, 8192, 1024), (20, 4096, 512)])
+@pytest.mark.parametrize("m,k,n", [(17, 5120, 512), (32, 5120, 768), (24, 9216, 512), (32, 8192, 1024), (20, 4096, 512),
+                                   (24, 3584, 18944), (32, 2560, 18432)])   # wide outputs: blocks of three pairs
 def test_lora_on_ten_wavefronts(oracle, m, k, n):
     """Up to 32 rows the blocks of a call with adapters may have ten wavefronts, in plans of one or two K slices:
     40 and 32 groups unsliced, 72 and 64 in two slices."""
