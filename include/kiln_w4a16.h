@@ -70,6 +70,7 @@ typedef int kiln_marlin_status_t;
  * with the same name and argument order.  Differences, all documented:
  *   - A and C are bf16 (the reference wrapper's two casts, lib.rs:169,269, go away);
  *   - B and s are in the tile layout;
+ *   - A, B, C, s and `workspace` must be 16-byte aligned (KILN_W4A16_ERR_ARGUMENT otherwise);
  *   - `workspace` must hold kiln_w4a16_workspace_bytes(m, n, k) bytes (with overrides:
  *     kiln_w4a16_workspace_bytes_tuned), its first kiln_w4a16_workspace_zeroed_bytes()
  *     bytes zero on first use; every call leaves that prefix zero again (the

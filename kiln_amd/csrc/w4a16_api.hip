@@ -873,6 +873,9 @@ kiln_marlin_status_t gemm_any(const void *A, const void *B, void *C, const void 
     if (thread_n > 0 && thread_n % 16 != 0) return KILN_W4A16_ERR_PROB_SHAPE;
     if (prob_m == 0 || prob_n == 0 || prob_k == 0) return KILN_W4A16_OK;  // marlin_kernel.cu:772-773
     if (!A || !B || !C || !s || !workspace) return KILN_W4A16_ERR_ARGUMENT;
+    // the kernels move every operand in 16-byte pieces (rows of A and C are multiples of 256 and 512 bytes)
+    for (const void *p : {A, B, static_cast<const void *>(C), s, static_cast<const void *>(workspace)})
+        if (reinterpret_cast<uintptr_t>(p) % 16 != 0) return KILN_W4A16_ERR_ARGUMENT;
 
     const int cus = sms > 0 ? sms : compute_units(dev);
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
@@ -1298,6 +1301,7 @@ kiln_marlin_status_t kiln_w4a16_gemm_lora(const void *A, const void *B, void *C,
     if (sum != r_total) return KILN_W4A16_ERR_ARGUMENT;
     if (prob_m == 0 || prob_n == 0 || prob_k == 0) return KILN_W4A16_OK;
     if (!A || !B || !C || !s || !workspace || !lora_a || !lora_b) return KILN_W4A16_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(lora_a) % 16 != 0 || reinterpret_cast<uintptr_t>(lora_b) % 16 != 0) return KILN_W4A16_ERR_ARGUMENT;
 
     const LoraSpec lora{lora_a, lora_b, r_total, n_adapters, ranks, scales};
     return gemm_any(A, B, C, s, prob_m, prob_n, prob_k, workspace, groupsize, dev, stream, -1, -1, -1, &lora);
@@ -1328,6 +1332,7 @@ kiln_marlin_status_t kiln_w4a16_gemm_swiglu_lora(const void *A, const void *B, v
     if (sum != r_total) return KILN_W4A16_ERR_ARGUMENT;
     if (prob_m == 0 || n_out == 0 || prob_k == 0) return KILN_W4A16_OK;
     if (!A || !B || !C || !s || !workspace || !lora_a || !lora_b) return KILN_W4A16_ERR_ARGUMENT;
+    if (reinterpret_cast<uintptr_t>(lora_a) % 16 != 0 || reinterpret_cast<uintptr_t>(lora_b) % 16 != 0) return KILN_W4A16_ERR_ARGUMENT;
     // the low-rank term lands on the f32 sums of gate and up before silu(gate) * up is formed; lora_b's rows
     // follow the packed columns, so an adapter of gate and one of up are two column blocks of one stacked B
     const LoraSpec lora{lora_a, lora_b, r_total, n_adapters, ranks, scales};

@@ -319,6 +319,35 @@ def test_matmul_bf16_rank3_and_pack_from_bf16(oracle):
         marlin_proj.matmul_bf16(torch.zeros(4, 128, dtype=torch.bfloat16, device="cuda"), proj)
 
 
+def test_operands_off_the_16_byte_grid_are_refused():
+    """The C entry itself (the wrappers make their tensors contiguous and torch aligns them): an A, C or workspace
+    that is not 16-byte aligned is an argument error, before anything is launched."""
+    from kiln_amd import _lib
+    L = _lib.load()
+    m, k, n = 4, 256, 256
+    x = torch.zeros(m * k + 8, dtype=torch.bfloat16, device="cuda")
+    b = torch.zeros(k // 16, 2 * n, dtype=torch.int32, device="cuda")
+    s = torch.ones(k // 128, n, dtype=torch.float16, device="cuda")
+    y = torch.zeros(m * n + 8, dtype=torch.bfloat16, device="cuda")
+    ws = torch.zeros(L.kiln_w4a16_workspace_bytes(m, n, k) + 64, dtype=torch.uint8, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    call = lambda xp, yp, wp: L.kiln_marlin_w4a16_gemm(xp, b.data_ptr(), yp, s.data_ptr(), m, n, k, wp, 128, 0, stream, -1, -1, -1, 16)
+    assert call(x.data_ptr(), y.data_ptr(), ws.data_ptr()) == 0
+    assert call(x.data_ptr() + 2, y.data_ptr(), ws.data_ptr()) == 4
+    assert call(x.data_ptr(), y.data_ptr() + 6, ws.data_ptr()) == 4
+    assert call(x.data_ptr(), y.data_ptr(), ws.data_ptr() + 8) == 4
+    assert call(x.data_ptr() + 16, y.data_ptr() + 16, ws.data_ptr() + 16) == 0
+    import ctypes
+    la = torch.zeros(8 * k + 8, dtype=torch.bfloat16, device="cuda")
+    lb = torch.zeros(n * 8 + 8, dtype=torch.bfloat16, device="cuda")
+    ranks, scales = (ctypes.c_int * 1)(8), (ctypes.c_float * 1)(1.0)
+    lora = lambda ap, bp: L.kiln_w4a16_gemm_lora(x.data_ptr(), b.data_ptr(), y.data_ptr(), s.data_ptr(), m, n, k, ws.data_ptr(), 128, 0,
+                                                 stream, ap, bp, 8, 1, ranks, scales)
+    assert lora(la.data_ptr(), lb.data_ptr()) == 0
+    assert lora(la.data_ptr() + 2, lb.data_ptr()) == 4 and lora(la.data_ptr(), lb.data_ptr() + 4) == 4
+    torch.cuda.synchronize()
+
+
 def test_wrapper_argument_checks_on_device():
     """lib.rs:112-166"""
     dev = "cuda"
